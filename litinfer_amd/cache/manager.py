@@ -156,6 +156,9 @@ class CacheManager:
             self._lib.li_book_destroy(self._book)
             self._book = None
             raise ValueError(err)
+        for gi, g in enumerate(self.groups):
+            if g.need.keep_first and self._lib.li_book_set_keep_first(self._book, gi, int(g.need.keep_first)) < 0:
+                raise ValueError(self._error())
         self._ints = (ctypes.c_int * max(ng, 1))()
         for gi, g in enumerate(self.groups):
             g.pool = PagePool(counts[gi], _borrowed=self._lib.li_book_pool(self._book, gi))

@@ -49,9 +49,11 @@ def architecture_name(cfg: Dict[str, Any]) -> str:
     archs = cfg.get("architectures")
     if isinstance(archs, list) and archs:
         return str(archs[0])
+    if isinstance(cfg.get("architecture"), str) and cfg["architecture"]:
+        return cfg["architecture"]
     if cfg.get("model_type"):
         return str(cfg["model_type"])
-    raise ValueError("config.json names no architecture (keys 'architectures', 'model_type')")
+    raise ValueError("config.json names no architecture (keys 'architectures', 'architecture', 'model_type')")
 
 
 def lookup(name: str) -> Architecture:

@@ -39,6 +39,9 @@ class ExecEntry:
     `cache_from` of the order (an earlier one) wrote."""
     layer: int
     cache_from: Optional[int] = None
+    # (i, k): before this entry runs, injection i of the model (`ModelSpec.injections`) acts on the
+    # residual stream for the k-th time (a part of category "injection": `forward(stream, ctx, k, embedding)`)
+    inject: Optional[Tuple[int, int]] = None
 
 
 @dataclass(frozen=True)
@@ -53,6 +56,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     eos_token_ids: Tuple[int, ...] = ()
+    injections: Tuple[PartSpec, ...] = ()
 
     def validate(self) -> None:
         if not self.layers:
@@ -63,6 +67,9 @@ class ModelSpec:
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"model spec: order[{i}] names layer {e.layer}, "
                                  f"there are {len(self.layers)}")
+            if e.inject is not None and not 0 <= e.inject[0] < len(self.injections):
+                raise ValueError(f"model spec: order[{i}] names injection {e.inject[0]}, "
+                                 f"there are {len(self.injections)}")
             if e.cache_from is not None:
                 if not 0 <= e.cache_from < i:
                     raise ValueError(f"model spec: order[{i}] reads the cache of entry "

@@ -373,3 +373,336 @@ extern "C" int li_rope_kv_store(void* qkv, int dtype, int row_stride, int nh, in
     else return LI_ERR_DTYPE;
     return li_launch_status();
 }
+
+// ============================================================================================
+// Parts that several designs share: a stream that takes a second gather and a vector, a norm whose
+// result is ADDED to the stream (a norm behind a sublayer), squared ReLU, a tanh-GELU gate times a
+// slice of a second embedding table, rotary tables from given frequencies, and the rotation of
+// neighbouring pairs.
+// ============================================================================================
+
+// out[t, :] += (table ? table[id(t), :] : 0) + (vec ? vec[:] : 0), all in float32; ids as in embedding_kernel
+template <typename T>
+__global__ void embedding_add_kernel(const int* __restrict__ ids, const int* __restrict__ id_src,
+                                     const int* __restrict__ feedback, const T* __restrict__ table,
+                                     const float* __restrict__ vec, float* __restrict__ out, int H, int V) {
+    const int t = blockIdx.x;
+    int id = -1;
+    if (table) {                                   // (without a table no ids are given)
+        id = ids[t];
+        if (id_src) {
+            const int src = id_src[t];
+            if (src >= 0) id = feedback[src];
+        }
+    }
+    float* o = out + (size_t)t * H;
+    const T* row = (table && id >= 0 && id < V) ? table + (size_t)id * H : nullptr;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+        float v = o[j];
+        if (row) v += load_as_float(row + j);
+        if (vec) v += vec[j];
+        o[j] = v;
+    }
+}
+
+extern "C" int li_embedding_add(const int* ids, const int* id_src, const int* feedback, const void* table,
+                                int table_dtype, const float* vec, float* out, int T, int H, int V, hipStream_t stream) {
+    if (T <= 0 || H <= 0 || (id_src && !feedback) || (table && !ids)) return LI_ERR_SIZE;
+    if (table_dtype == LI_F32)
+        embedding_add_kernel<float><<<T, 256, 0, stream>>>(ids, id_src, feedback, (const float*)table, vec, out, H, V);
+    else if (table_dtype == LI_BF16)
+        embedding_add_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, id_src, feedback, (const bf16_t*)table, vec, out, H, V);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// x[t, :] += y[t, :] / sqrt(mean(y^2) + eps) * w, and, where w2 is given, xn[t, :] = the RMS norm
+// of the NEW x with weights w2 and eps2 (the norm through which the stream is read next): one block a row.
+template <typename TO, int NT>
+__global__ __launch_bounds__(NT) void rmsnorm_add_kernel(const float* __restrict__ y, const float* __restrict__ w, float eps,
+                                                          float* __restrict__ x, const float* __restrict__ w2, float eps2,
+                                                          TO* __restrict__ xn, int H) {
+    __shared__ float red[NT / LI_WAVE];
+    const float* yr = y + (size_t)blockIdx.x * H;
+    float* xr = x + (size_t)blockIdx.x * H;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < H; j += NT) { const float v = yr[j]; ss += v * v; }
+    ss = block_sum<NT>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    float s2 = 0.f;
+    for (int j = threadIdx.x; j < H; j += NT) {
+        const float v = xr[j] + yr[j] * inv * w[j];
+        xr[j] = v;
+        s2 += v * v;
+    }
+    if (w2 == nullptr) return;
+    s2 = block_sum<NT>(s2, red);
+    const float inv2 = 1.0f / sqrtf(s2 / (float)H + eps2);
+    TO* o = xn + (size_t)blockIdx.x * H;
+    for (int j = threadIdx.x; j < H; j += NT) store_from_float(o + j, xr[j] * inv2 * w2[j]);     // (a thread reads back what it wrote)
+}
+
+extern "C" int li_rmsnorm_add(const float* y, const float* w, float eps, float* x, const float* w2, float eps2,
+                              void* xn, int xn_dtype, int T, int H, hipStream_t stream) {
+    if (T <= 0 || H <= 0) return LI_ERR_SIZE;
+    if (w2 && !xn) return LI_ERR_SIZE;
+    const bool wide = T < 256 && H > 1024;
+#define LI_RA(TO)                                                                                             \
+    {                                                                                                         \
+        if (wide) rmsnorm_add_kernel<TO, 1024><<<T, 1024, 0, stream>>>(y, w, eps, x, w2, eps2, (TO*)xn, H);   \
+        else rmsnorm_add_kernel<TO, 256><<<T, 256, 0, stream>>>(y, w, eps, x, w2, eps2, (TO*)xn, H);          \
+    }
+    if (!w2 || xn_dtype == LI_F32) LI_RA(float)
+    else if (xn_dtype == LI_BF16) LI_RA(bf16_t)
+    else return LI_ERR_DTYPE;
+#undef LI_RA
+    return li_launch_status();
+}
+
+// out = max(x, 0)^2
+template <typename TI, typename TO>
+__global__ void relu_squared_kernel(const TI* __restrict__ x, TO* __restrict__ out, long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float v = fmaxf(load_as_float(x + i), 0.f);
+        store_from_float(out + i, v * v);
+    }
+}
+
+extern "C" int li_relu_squared(const void* x, int x_dtype, void* out, int out_dtype, long n, hipStream_t stream) {
+    if (n <= 0) return LI_ERR_SIZE;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (x_dtype == LI_F32 && out_dtype == LI_F32) relu_squared_kernel<float, float><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, n);
+    else if (x_dtype == LI_F32 && out_dtype == LI_BF16) relu_squared_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>((const float*)x, (bf16_t*)out, n);
+    else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) relu_squared_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, n);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+__device__ __forceinline__ float gelu_tanh(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// out[t, j] = gelu_tanh(a[t, j]) * table[id(t), off + j], j < n; table rows have `row` elements
+template <typename TT, typename TO>
+__global__ void gelu_gate_rows_kernel(const float* __restrict__ a, const int* __restrict__ ids, const int* __restrict__ id_src,
+                                      const int* __restrict__ feedback, const TT* __restrict__ table, int row, int off, int V,
+                                      TO* __restrict__ out, int n) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id_src) {
+        const int src = id_src[t];
+        if (src >= 0) id = feedback[src];
+    }
+    const bool ok = id >= 0 && id < V;
+    const TT* e = table + (size_t)(ok ? id : 0) * row + off;
+    for (int j = threadIdx.x; j < n; j += blockDim.x)
+        store_from_float(out + (size_t)t * n + j, ok ? gelu_tanh(a[(size_t)t * n + j]) * load_as_float(e + j) : 0.f);
+}
+
+extern "C" int li_gelu_gate_rows(const float* a, const int* ids, const int* id_src, const int* feedback, const void* table,
+                                 int table_dtype, int row, int off, int V, void* out, int out_dtype, int T, int n,
+                                 hipStream_t stream) {
+    if (T <= 0 || n <= 0 || off < 0 || off + n > row || (id_src && !feedback)) return LI_ERR_SIZE;
+    const int nt = n >= 256 ? 256 : 64;
+#define LI_GG(TT, TO) gelu_gate_rows_kernel<TT, TO><<<T, nt, 0, stream>>>(a, ids, id_src, feedback, (const TT*)table, row, off, V, (TO*)out, n)
+    if (table_dtype == LI_F32 && out_dtype == LI_F32) LI_GG(float, float);
+    else if (table_dtype == LI_BF16 && out_dtype == LI_BF16) LI_GG(bf16_t, bf16_t);
+    else if (table_dtype == LI_BF16 && out_dtype == LI_F32) LI_GG(bf16_t, float);
+    else if (table_dtype == LI_F32 && out_dtype == LI_BF16) LI_GG(float, bf16_t);
+    else return LI_ERR_DTYPE;
+#undef LI_GG
+    return li_launch_status();
+}
+
+// cos/sin [T, n] of angle = float(pos[t]) * freq[i], each times `amp`: the frequencies are given
+// (whatever scaling they went through on the host), the product and the functions are float32
+__global__ void rope_freq_table_kernel(const int* __restrict__ pos, const float* __restrict__ freq, int n, float amp,
+                                       float* __restrict__ cosv, float* __restrict__ sinv, int T) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long)T * n) return;
+    const int t = (int)(idx / n), i = (int)(idx % n);
+    const float ang = (float)pos[t] * freq[i];
+    cosv[idx] = cosf(ang) * amp;
+    sinv[idx] = sinf(ang) * amp;
+}
+
+extern "C" int li_rope_freq_table(const int* pos, const float* freq, int n, float amp, float* cosv, float* sinv, int T,
+                                  hipStream_t stream) {
+    if (T <= 0 || n <= 0) return LI_ERR_SIZE;
+    const long total = (long)T * n;
+    rope_freq_table_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(pos, freq, n, amp, cosv, sinv, T);
+    return li_launch_status();
+}
+
+// neighbouring pairs: (u, v) = (x[2i], x[2i+1]) -> (u cos - v sin, v cos + u sin)
+__device__ __forceinline__ void rotate_pair(float u, float v, float c, float s, float& ru, float& rv) {
+    ru = fmaf(u, c, -__fmul_rn(v, s));
+    rv = fmaf(v, c, __fmul_rn(u, s));
+}
+
+// in place, heads 0..n_heads-1 of every row (head h at columns h * head_dim ..), the first rotary_dim of each
+template <typename T>
+__global__ void rope_pairs_apply_kernel(T* __restrict__ x, int row_stride, int n_heads, int head_dim, int rotary_dim,
+                                        const float* __restrict__ cosv, const float* __restrict__ sinv) {
+    const int t = blockIdx.x, half = rotary_dim / 2;
+    T* row = x + (size_t)t * row_stride;
+    for (int u = threadIdx.x; u < n_heads * half; u += blockDim.x) {
+        const int h = u / half, i = u % half;
+        T* p = row + (size_t)h * head_dim + 2 * i;
+        float a, b;
+        rotate_pair(load_as_float(p), load_as_float(p + 1), cosv[(size_t)t * half + i], sinv[(size_t)t * half + i], a, b);
+        store_from_float(p, a);
+        store_from_float(p + 1, b);
+    }
+}
+
+extern "C" int li_rope_pairs_apply(void* x, int dtype, int row_stride, int n_heads, int head_dim, int rotary_dim,
+                                   const float* cosv, const float* sinv, int T, hipStream_t stream) {
+    if (T <= 0 || n_heads <= 0 || rotary_dim <= 0 || (rotary_dim & 1) || rotary_dim > head_dim) return LI_ERR_SIZE;
+    if (dtype == LI_F32) rope_pairs_apply_kernel<float><<<T, 256, 0, stream>>>((float*)x, row_stride, n_heads, head_dim, rotary_dim, cosv, sinv);
+    else if (dtype == LI_BF16) rope_pairs_apply_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)x, row_stride, n_heads, head_dim, rotary_dim, cosv, sinv);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// The step between the packed q/k/v projection (float32 rows [q | k | v]) and the attention, for a mixer that
+// norms the WHOLE query projection and the WHOLE key projection (all heads at once, before they are split) and
+// rotates neighbouring pairs: q is normed and rotated in place (it stays float32), k is normed, rotated and
+// written to its page slot, v is copied to its page slot.  wq / wk null: no norm.  One block a token.
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void qk_norm_pairs_store_kernel(
+    float* __restrict__ qkv, int row_stride, int nh, int nkv, int dk, int dv, int rotary_dim,
+    const float* __restrict__ wq, const float* __restrict__ wk, float eps,
+    const float* __restrict__ cosv, const float* __restrict__ sinv, const int* __restrict__ slot_map,
+    T* __restrict__ kc, T* __restrict__ vc, int page_size, int store) {
+    __shared__ float red[NT / LI_WAVE];
+    const int t = blockIdx.x, half = rotary_dim / 2;
+    float* q = qkv + (size_t)t * row_stride;
+    float* k = q + (size_t)nh * dk;
+    const float* v = k + (size_t)nkv * dk;
+    const int nq = nh * dk, nk = nkv * dk;
+    float inv_q = 1.f, inv_k = 1.f;
+    if (wq) {
+        float s = 0.f;
+        for (int j = threadIdx.x; j < nq; j += NT) s += q[j] * q[j];
+        s = block_sum<NT>(s, red);
+        inv_q = 1.0f / sqrtf(s / (float)nq + eps);
+    }
+    if (wk && store) {
+        float s = 0.f;
+        for (int j = threadIdx.x; j < nk; j += NT) s += k[j] * k[j];
+        s = block_sum<NT>(s, red);
+        inv_k = 1.0f / sqrtf(s / (float)nk + eps);
+    }
+    const float* c = cosv + (size_t)t * half;
+    const float* sn = sinv + (size_t)t * half;
+    const int units = half + (dk - rotary_dim);            // per head: the pairs, then the columns that are not rotated
+    for (int u = threadIdx.x; u < nh * units; u += NT) {
+        const int h = u / units, i = u % units;
+        if (i < half) {
+            const int j = h * dk + 2 * i;
+            const float a = wq ? q[j] * inv_q * wq[j] : q[j], b = wq ? q[j + 1] * inv_q * wq[j + 1] : q[j + 1];
+            float ra, rb;
+            rotate_pair(a, b, c[i], sn[i], ra, rb);
+            q[j] = ra; q[j + 1] = rb;
+        } else if (wq) {
+            const int j = h * dk + rotary_dim + (i - half);
+            q[j] = q[j] * inv_q * wq[j];
+        }
+    }
+    if (!store) return;
+    const int slot = slot_map[t], page = slot / page_size, off = slot % page_size;
+    for (int u = threadIdx.x; u < nkv * units; u += NT) {
+        const int h = u / units, i = u % units;
+        T* dst = kc + ((size_t)(page * nkv + h) * page_size + off) * dk;
+        if (i < half) {
+            const int j = h * dk + 2 * i;
+            const float a = wk ? k[j] * inv_k * wk[j] : k[j], b = wk ? k[j + 1] * inv_k * wk[j + 1] : k[j + 1];
+            float ra, rb;
+            rotate_pair(a, b, c[i], sn[i], ra, rb);
+            store_from_float(dst + 2 * i, ra);
+            store_from_float(dst + 2 * i + 1, rb);
+        } else {
+            const int d = rotary_dim + (i - half), j = h * dk + d;
+            store_from_float(dst + d, wk ? k[j] * inv_k * wk[j] : k[j]);
+        }
+    }
+    for (int u = threadIdx.x; u < nkv * dv; u += NT) {
+        const int h = u / dv, d = u % dv;
+        store_from_float(vc + ((size_t)(page * nkv + h) * page_size + off) * dv + d, v[u]);
+    }
+}
+
+extern "C" int li_qk_norm_pairs_store(float* qkv, int row_stride, int nh, int nkv, int dk, int dv, int rotary_dim,
+                                      const float* wq, const float* wk, float eps, const float* cosv, const float* sinv,
+                                      const int* slot_map, void* kc, void* vc, int cache_dtype, int page_size, int store,
+                                      int T, hipStream_t stream) {
+    if (T <= 0 || nh <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > dk ||
+        row_stride < nh * dk + nkv * (dk + dv) || page_size <= 0)
+        return LI_ERR_SIZE;
+    if (cache_dtype == LI_F32)
+        qk_norm_pairs_store_kernel<float, 256><<<T, 256, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps,
+                                                                      cosv, sinv, slot_map, (float*)kc, (float*)vc, page_size, store);
+    else if (cache_dtype == LI_BF16)
+        qk_norm_pairs_store_kernel<bf16_t, 256><<<T, 256, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps,
+                                                                       cosv, sinv, slot_map, (bf16_t*)kc, (bf16_t*)vc, page_size, store);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// The same step for attention over a compressed cache.  A row of `qd` (float32) is [q | down]: q holds nh heads of
+// (dn + dr) columns, the last dr of each rotated; down holds `rank` latent columns and dr columns of one rotated key
+// part that all heads share.  The latent is RMS-normed (weights wc) and written to columns 0..rank-1 of the token's
+// page row, the rotated shared part behind it; the rotated part of every query head goes to columns rank.. of
+// that head's row in `qfull` (float32 rows of nh x (rank + dr): the first `rank` columns are filled by the product
+// with the keys' expansion matrix afterwards).
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void latent_norm_pairs_store_kernel(
+    const float* __restrict__ qd, int row_stride, int nh, int dn, int dr, int rank, const float* __restrict__ wc, float eps,
+    const float* __restrict__ cosv, const float* __restrict__ sinv, const int* __restrict__ slot_map,
+    T* __restrict__ cache, float* __restrict__ qfull, int store) {
+    __shared__ float red[NT / LI_WAVE];
+    const int t = blockIdx.x, half = dr / 2;
+    const float* q = qd + (size_t)t * row_stride;
+    const float* down = q + (size_t)nh * (dn + dr);
+    const float* c = cosv + (size_t)t * half;
+    const float* sn = sinv + (size_t)t * half;
+    float* qf = qfull + (size_t)t * nh * (rank + dr);
+    for (int u = threadIdx.x; u < nh * half; u += NT) {
+        const int h = u / half, i = u % half;
+        const float* src = q + (size_t)h * (dn + dr) + dn + 2 * i;
+        float ra, rb;
+        rotate_pair(src[0], src[1], c[i], sn[i], ra, rb);
+        float* dst = qf + (size_t)h * (rank + dr) + rank + 2 * i;
+        dst[0] = ra; dst[1] = rb;
+    }
+    if (!store) return;
+    float s = 0.f;
+    for (int j = threadIdx.x; j < rank; j += NT) s += down[j] * down[j];
+    s = block_sum<NT>(s, red);
+    const float inv = 1.0f / sqrtf(s / (float)rank + eps);
+    T* row = cache + (size_t)slot_map[t] * (rank + dr);
+    for (int j = threadIdx.x; j < rank; j += NT) store_from_float(row + j, down[j] * inv * wc[j]);
+    for (int i = threadIdx.x; i < half; i += NT) {
+        float ra, rb;
+        rotate_pair(down[rank + 2 * i], down[rank + 2 * i + 1], c[i], sn[i], ra, rb);
+        store_from_float(row + rank + 2 * i, ra);
+        store_from_float(row + rank + 2 * i + 1, rb);
+    }
+}
+
+extern "C" int li_latent_norm_pairs_store(const float* qd, int row_stride, int nh, int dn, int dr, int rank, const float* wc,
+                                          float eps, const float* cosv, const float* sinv, const int* slot_map, void* cache,
+                                          int cache_dtype, float* qfull, int store, int T, hipStream_t stream) {
+    if (T <= 0 || nh <= 0 || dn < 0 || dr <= 0 || (dr & 1) || rank <= 0 || row_stride < nh * (dn + dr) + rank + dr)
+        return LI_ERR_SIZE;
+    if (cache_dtype == LI_F32)
+        latent_norm_pairs_store_kernel<float, 256><<<T, 256, 0, stream>>>(qd, row_stride, nh, dn, dr, rank, wc, eps, cosv, sinv,
+                                                                          slot_map, (float*)cache, qfull, store);
+    else if (cache_dtype == LI_BF16)
+        latent_norm_pairs_store_kernel<bf16_t, 256><<<T, 256, 0, stream>>>(qd, row_stride, nh, dn, dr, rank, wc, eps, cosv, sinv,
+                                                                           slot_map, (bf16_t*)cache, qfull, store);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}

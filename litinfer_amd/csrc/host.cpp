@@ -86,6 +86,7 @@ struct Request {
 struct Book {
     int page_size = 0, max_seqs = 0;
     std::vector<int> windows;                  // per group, 0 = all keys
+    std::vector<int> keep_first;               // per group: a windowed group never gives back the pages of its first so many positions
     std::vector<Pool> pools;
     std::vector<int> free_slots;
     std::unordered_map<int64_t, Request> requests;
@@ -147,6 +148,7 @@ void* li_book_create(int page_size, int max_seqs, int ngroups, const int* window
     if (page_size <= 0) { b->error = "cache: page_size must be positive"; return b; }
     if (max_seqs <= 0 || ngroups < 0) { b->error = "cache: max_seqs must be positive"; return b; }
     b->windows.assign(windows, windows + ngroups);
+    b->keep_first.assign(ngroups, 0);
     b->pools.resize(ngroups);
     size_t at = 0;
     for (int g = 0; g < ngroups; ++g) {
@@ -159,6 +161,15 @@ void* li_book_create(int page_size, int max_seqs, int ngroups, const int* window
     b->free_slots.resize(max_seqs);
     for (int i = 0; i < max_seqs; ++i) b->free_slots[i] = max_seqs - 1 - i;
     return b;
+}
+// A windowed group whose queries also see the first n positions of their request whatever the
+// distance: the pages of those positions stay with the request until it ends.
+int li_book_set_keep_first(void* vb, int g, int n) {
+    Book* b = (Book*)vb;
+    if (g < 0 || g >= (int)b->pools.size() || n < 0) return b->fail(ERR_ARG, "cache: keep_first of an unknown group");
+    if (!b->requests.empty()) return b->fail(ERR_LIVE, "cache: keep_first is set before any request is admitted");
+    b->keep_first[g] = n;
+    return 0;
 }
 void li_book_destroy(void* b) { delete (Book*)b; }
 const char* li_book_error(void* b) { return ((Book*)b)->error.c_str(); }
@@ -311,7 +322,8 @@ int li_book_commit(void* vb, int64_t h, int n_new) {
     for (size_t g = 0; g < b->pools.size(); ++g) {
         if (b->windows[g] <= 0) continue;
         const int keep_from = std::min(b->first_needed_block((int)g, r->cached), (int)r->tables[g].size());
-        for (int blk = r->first_live[g]; blk < keep_from; ++blk)
+        const int kept = (b->keep_first[g] + b->page_size - 1) / b->page_size;     // blocks that every later query still sees
+        for (int blk = std::max(r->first_live[g], kept); blk < keep_from; ++blk)
             if (r->tables[g][blk] >= 0) {
                 const int rc = b->pools[g].release(r->tables[g][blk]);
                 if (rc < 0) return b->fail(rc, b->pools[g].error);

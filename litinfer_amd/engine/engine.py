@@ -174,7 +174,8 @@ class Engine:
             per_seq = -(-self.spec.max_positions // P)
             full = per_seq * self.max_seqs
             pages = [full if g.window <= 0 else
-                     min(full, self.max_seqs * (-(-g.window // P) + 2) + -(-self.step_tokens // P)) for g in groups]
+                     min(full, self.max_seqs * (-(-g.window // P) + 2 + -(-g.keep_first // P)) + -(-self.step_tokens // P))
+                     for g in groups]
             if self.rt.device.type == "cuda" and groups:
                 free, _ = torch.cuda.mem_get_info(self.rt.device)
                 bpp = [max(1, b) for b in self._group_page_bytes()]

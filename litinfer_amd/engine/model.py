@@ -22,20 +22,22 @@ class Model:
         self.layers = [build_part("block", PartSpec(l.block), rt, parts=l.parts) for l in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm, rt)
         self.head = build_part("head", spec.head, rt)
+        self.injections = [build_part("injection", s, rt) for s in spec.injections]
         self.order = list(spec.order)
+        self.tap = None                              # a callable (entry number, float32 stream [T, H]) for whoever debugs layers
         self._batch_needs = None
 
     # ---- weights ----------------------------------------------------------
     def expected_params(self) -> Dict[str, ParamSpec]:
         e: Dict[str, ParamSpec] = {}
-        for p in (self.embedding, *self.layers, self.final_norm, self.head):
+        for p in (self.embedding, *self.layers, *self.injections, self.final_norm, self.head):
             e.update(p.expected_params())
         return e
 
     def load_params(self, get) -> None:
         self._batch_needs = None                     # parts may answer differently once they hold their tensors
         self.embedding.load_params(get)
-        for layer in self.layers:
+        for layer in (*self.layers, *self.injections):
             layer.load_params(get)
         self.final_norm.load_params(get)
         self.head.load_params(get, tied_table=getattr(self.embedding, "table", None))
@@ -61,14 +63,14 @@ class Model:
         if self._batch_needs is None:
             from ..parts.base import BatchNeeds
             needs = BatchNeeds()
-            for p in (self.embedding, *self.layers, self.final_norm, self.head):
+            for p in (self.embedding, *self.layers, *self.injections, self.final_norm, self.head):
                 needs = needs.merged(p.batch_needs())
             self._batch_needs = needs
         return self._batch_needs
 
     @property
     def graph_safe(self) -> bool:
-        return all(p.graph_safe for p in (self.embedding, *self.layers, self.final_norm, self.head))
+        return all(p.graph_safe for p in (self.embedding, *self.layers, *self.injections, self.final_norm, self.head))
 
     # ---- cache ------------------------------------------------------------
     def cache_needs(self) -> Tuple[List[object], List[Optional[int]]]:
@@ -84,11 +86,17 @@ class Model:
         x = ctx.ws.buffer("model.residual", (ctx.num_tokens, h), torch.float32)
         self.embedding.forward(ctx.ids, x, ctx.id_src, ctx.feedback)
         stream = ResidualStream(x, ctx.ws)
+        stream.ws_dtype = self.rt.dtype
         for i, e in enumerate(self.order):
-            # the block is told through which norm the next one reads what it leaves
-            follower = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else None
+            if e.inject is not None:
+                self.injections[e.inject[0]].forward(stream, ctx, e.inject[1], self.embedding)
+            # the block is told through which norm the next one reads what it leaves (if nothing is added between them)
+            nxt = self.order[i + 1] if i + 1 < len(self.order) else None
+            follower = self.layers[nxt.layer] if nxt is not None and nxt.inject is None else None
             stream.next_norm = follower.first_norm() if follower is not None else None
             self.layers[e.layer].forward(stream, ctx, cache.view(i))
+            if self.tap is not None:
+                self.tap(i, stream.x)
         x = stream.tensor()
         if ctx.num_want == 0:
             return None

@@ -32,7 +32,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="the most tokens live requests hold at any time (each rounded up to the page size)")
     ap.add_argument("--page-size", type=int, default=16)
-    ap.add_argument("--max-seqs", type=int, default=16, help="requests that may be live at a time")
+    ap.add_argument("--max-seqs", type=int, default=4, help="requests that may be live at a time (state slots)")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--page-order-seed", "--shuffle-pages", dest="page_order_seed", type=int, default=None,
                     help="shuffle the order in which free pages are handed out, so that block tables are not contiguous")
@@ -48,11 +48,8 @@ def main(argv=None) -> int:
     import numpy as np
     import torch                                   # noqa: F401
     from . import Engine, StepEntry
-    from ..kernels import build
-    missing = [m for m in build.MODULES if build.find_built(m) is None]
-    if missing:
-        _log(f"building the HIP kernels ({', '.join(missing)}) ...")
-        build.build_all(verbose=True, force=False)
+    # (a kernel library that is not built yet is compiled when the model first calls into it: only
+    # what this model needs)
     _log(f"loading {args.model} as {args.dtype} ...")
     pages = -(-max(1, args.max_tokens) // args.page_size)
     engine = Engine.from_dir(args.model, dtype=args.dtype, device=args.device, page_size=args.page_size,

@@ -164,7 +164,7 @@ class Scheduler:
         need = self.cache.pages_needed(None, len(prompt) + max_new_tokens - 1, cached=0)
         for g, n in zip(self.cache.groups, need):
             if g.need.window > 0:                      # there a request goes on token by token if it must
-                n = min(n, -(-g.need.window // self.cache.page_size) + 1)
+                n = min(n, -(-g.need.window // self.cache.page_size) + 1 + -(-g.need.keep_first // self.cache.page_size))
             if n > g.pool.capacity:
                 raise ValueError(f"add_request: the request needs {n} cache pages, the pool has "
                                  f"{g.pool.capacity}: it could never run")
@@ -221,7 +221,8 @@ class Scheduler:
         than that serves one request at a time, in shorter portions."""
         P = self.cache.page_size
         portion = self.chunk_size if portion is None else portion
-        caps = [min(-(-(g.need.window - 1 + portion) // P) + 1, g.pool.capacity) if g.need.window > 0 else None
+        caps = [min(-(-(g.need.window - 1 + portion) // P) + 1 + -(-g.need.keep_first // P), g.pool.capacity)
+                if g.need.window > 0 else None
                 for g in self.cache.groups]
         if all(c is None for c in caps):
             return need

@@ -36,6 +36,18 @@ _SIGNATURES = {
         "li_rope_apply": [P, I, I, I, I, I, P, P, I],
         "li_kv_store": [P, I, I, I, I, I, P, P, P, I, I, I],
         "li_rope_kv_store": [P, I, I, I, I, I, I, P, P, P, P, P, I, I, I],
+        "li_embedding_add": [P, P, P, P, I, P, P, I, I, I],
+        "li_rmsnorm_add": [P, P, F, P, P, F, P, I, I, I],
+        "li_relu_squared": [P, I, P, I, L],
+        "li_gelu_gate_rows": [P, P, P, P, P, I, I, I, I, P, I, I, I],
+        "li_rope_freq_table": [P, P, I, F, P, P, I],
+        "li_rope_pairs_apply": [P, I, I, I, I, I, P, P, I],
+        "li_qk_norm_pairs_store": [P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, I],
+        "li_latent_norm_pairs_store": [P, I, I, I, I, I, P, F, P, P, P, P, I, P, I, I],
+    },
+    "attention_masked": {
+        "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, I, F, F],
+        "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I],
     },
     "gemm": {
         "li_linear": [P, P, P, P, I, I, I, I, I, I, P, L],
@@ -308,6 +320,209 @@ def rope_kv_store(qkv: torch.Tensor, nh: int, nkv: int, dh: int, rotary_dim: int
         _run("elementwise", "li_rope_kv_store", qkv.data_ptr(), _DT[qkv.dtype], qkv.stride(0), nh, nkv,
              dh, rotary_dim, cos.data_ptr(), sin.data_ptr(), slot_map.data_ptr(), k.data_ptr(),
              v.data_ptr(), page_size, k.shape[0], t)
+
+
+def _ids_ok(ids, id_src, feedback, t) -> bool:
+    return (ids.dtype is torch.int32 and ids.numel() == t and ids.is_contiguous()
+            and (id_src is None or (feedback is not None and id_src.dtype is torch.int32 and id_src.numel() == t
+                                    and id_src.is_contiguous() and feedback.dtype is torch.int32
+                                    and feedback.is_contiguous())))
+
+
+def embedding_add(out: torch.Tensor, ids: Optional[torch.Tensor] = None, table: Optional[torch.Tensor] = None,
+                  vec: Optional[torch.Tensor] = None, id_src: Optional[torch.Tensor] = None,
+                  feedback: Optional[torch.Tensor] = None) -> None:
+    """out[t, :] += table[id(t), :] (if a table is given) + vec[:] (if given), in float32; ids as in
+    `embedding` (an id outside the table adds nothing)."""
+    _gpu(out, ids, table, vec, id_src, feedback)
+    t, h = out.shape
+    _chk(out.dtype is torch.float32 and out.is_contiguous(), "embedding_add: out must be float32")
+    _chk(table is None or (ids is not None and table.dim() == 2 and table.shape[1] == h and table.is_contiguous()
+                           and table.dtype in _DT and _ids_ok(ids, id_src, feedback, t)), "embedding_add: table, ids")
+    _chk(vec is None or (vec.dtype is torch.float32 and vec.numel() == h and vec.is_contiguous()), "embedding_add: vec")
+    if t and (table is not None or vec is not None):
+        if table is None:
+            ids = id_src = feedback = None
+        _run("elementwise", "li_embedding_add", 0 if ids is None else ids.data_ptr(), 0 if id_src is None else id_src.data_ptr(),
+             0 if id_src is None else feedback.data_ptr(), 0 if table is None else table.data_ptr(),
+             _DT[table.dtype] if table is not None else 0, 0 if vec is None else vec.data_ptr(), out.data_ptr(), t, h,
+             table.shape[0] if table is not None else 0)
+
+
+def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch.Tensor,
+                next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
+                next_out: Optional[torch.Tensor] = None) -> None:
+    """x += y / sqrt(mean(y^2) + eps) * weight, row by row, in float32; with `next_weight` also
+    next_out = the RMS norm of the new x with those weights and `next_eps`."""
+    _gpu(y, weight, x, next_weight, next_out)
+    _chk(y.dim() == 2 and y.shape == x.shape and y.is_contiguous() and x.is_contiguous()
+         and y.dtype is torch.float32 and x.dtype is torch.float32, "rmsnorm_add: y and x must be contiguous float32 [T, H]")
+    h = x.shape[1]
+    _chk(weight.dtype is torch.float32 and weight.numel() == h and weight.is_contiguous(), "rmsnorm_add: weight")
+    if next_weight is not None:
+        _chk(next_out is not None and next_out.shape == x.shape and next_out.is_contiguous() and next_out.dtype in _DT
+             and next_weight.dtype is torch.float32 and next_weight.numel() == h and next_weight.is_contiguous(),
+             "rmsnorm_add: the next norm's weight and out")
+    if x.shape[0]:
+        _run("elementwise", "li_rmsnorm_add", y.data_ptr(), weight.data_ptr(), float(eps), x.data_ptr(),
+             0 if next_weight is None else next_weight.data_ptr(), float(next_eps),
+             0 if next_weight is None else next_out.data_ptr(), _DT[next_out.dtype] if next_weight is not None else 0,
+             x.shape[0], h)
+
+
+def relu_squared(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = max(x, 0)^2."""
+    _gpu(x, out)
+    _chk(x.shape == out.shape and x.is_contiguous() and out.is_contiguous() and x.dtype in _DT and out.dtype in _DT
+         and (x.dtype is torch.float32 or out.dtype is x.dtype), "relu_squared: x, out")
+    if x.numel():
+        _run("elementwise", "li_relu_squared", x.data_ptr(), _DT[x.dtype], out.data_ptr(), _DT[out.dtype], x.numel())
+
+
+def gelu_gate_rows(a: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, offset: int, out: torch.Tensor,
+                   id_src: Optional[torch.Tensor] = None, feedback: Optional[torch.Tensor] = None) -> None:
+    """out[t, j] = gelu_tanh(a[t, j]) * table[id(t), offset + j]."""
+    _gpu(a, ids, table, out, id_src, feedback)
+    t, n = a.shape
+    _chk(a.dtype is torch.float32 and a.is_contiguous() and out.shape == a.shape and out.is_contiguous()
+         and out.dtype in _DT, "gelu_gate_rows: a float32 [T, n], out [T, n]")
+    _chk(table.dim() == 2 and table.is_contiguous() and table.dtype in _DT and 0 <= offset
+         and offset + n <= table.shape[1] and _ids_ok(ids, id_src, feedback, t), "gelu_gate_rows: table, ids")
+    if t:
+        _run("elementwise", "li_gelu_gate_rows", a.data_ptr(), ids.data_ptr(), 0 if id_src is None else id_src.data_ptr(),
+             0 if id_src is None else feedback.data_ptr(), table.data_ptr(), _DT[table.dtype], table.shape[1], int(offset),
+             table.shape[0], out.data_ptr(), _DT[out.dtype], t, n)
+
+
+def rope_freq_table(positions: torch.Tensor, freq: torch.Tensor, amplitude: float, cos: torch.Tensor,
+                    sin: torch.Tensor) -> None:
+    """cos/sin [T, n] of angle = float(pos) * freq[i], times `amplitude`, in float32."""
+    _gpu(positions, freq, cos, sin)
+    t, n = positions.numel(), freq.numel()
+    _chk(positions.dtype is torch.int32 and positions.is_contiguous() and freq.dtype is torch.float32
+         and freq.is_contiguous(), "rope_freq_table: positions, freq")
+    _chk(cos.shape == (t, n) and sin.shape == cos.shape and cos.is_contiguous() and sin.is_contiguous()
+         and cos.dtype is torch.float32 and sin.dtype is torch.float32, "rope_freq_table: cos, sin")
+    if t:
+        _run("elementwise", "li_rope_freq_table", positions.data_ptr(), freq.data_ptr(), n, float(amplitude),
+             cos.data_ptr(), sin.data_ptr(), t)
+
+
+def rope_pairs_apply(qkv: torch.Tensor, n_heads: int, head_dim: int, rotary_dim: int, cos: torch.Tensor,
+                     sin: torch.Tensor) -> None:
+    """Rotate heads 0..n_heads-1 of every row in place, neighbouring columns (2i, 2i+1) forming a pair."""
+    _gpu(qkv, cos, sin)
+    _check_qkv(qkv, n_heads, head_dim)
+    t = qkv.shape[0]
+    _chk(cos.shape == (t, rotary_dim // 2) and sin.shape == cos.shape and rotary_dim <= head_dim
+         and cos.dtype is torch.float32 and cos.is_contiguous() and sin.is_contiguous(), "rope_pairs_apply: tables")
+    if t:
+        _run("elementwise", "li_rope_pairs_apply", qkv.data_ptr(), _DT[qkv.dtype], qkv.stride(0), n_heads, head_dim,
+             rotary_dim, cos.data_ptr(), sin.data_ptr(), t)
+
+
+def _check_tables(what, t, rotary_dim, cos, sin, slot_map):
+    _chk(cos.shape == (t, rotary_dim // 2) and sin.shape == cos.shape and cos.dtype is torch.float32
+         and sin.dtype is torch.float32 and cos.is_contiguous() and sin.is_contiguous(), f"{what}: tables")
+    _chk(slot_map is None or (slot_map.dtype is torch.int32 and slot_map.numel() == t and slot_map.is_contiguous()),
+         f"{what}: slot_map")
+
+
+def qk_norm_pairs_store(qkv: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, rotary_dim: int,
+                        wq: Optional[torch.Tensor], wk: Optional[torch.Tensor], eps: float, cos: torch.Tensor,
+                        sin: torch.Tensor, slot_map: Optional[torch.Tensor], k: Optional[torch.Tensor],
+                        v: Optional[torch.Tensor], page_size: int) -> None:
+    """qkv float32 rows [q (nh*dk) | k (nkv*dk) | v (nkv*dv)].  q and k are RMS-normed over their WHOLE
+    width (weights wq, wk; None: no norm), their heads' first `rotary_dim` columns rotated in neighbouring
+    pairs; q stays in place, k and v go to their page slots (k None: only q is prepared)."""
+    _gpu(qkv, wq, wk, cos, sin, slot_map, k, v)
+    t = qkv.shape[0]
+    _chk(_rows_ok(qkv) and qkv.dtype is torch.float32 and qkv.shape[1] >= nh * dk + nkv * (dk + dv),
+         "qk_norm_pairs_store: qkv must be float32 rows of q, k and v")
+    _chk(rotary_dim % 2 == 0 and 0 <= rotary_dim <= dk, "qk_norm_pairs_store: rotary_dim")
+    _check_tables("qk_norm_pairs_store", t, rotary_dim, cos, sin, slot_map if k is not None else None)
+    for w_, n_ in ((wq, nh * dk), (wk, nkv * dk)):
+        _chk(w_ is None or (w_.dtype is torch.float32 and w_.numel() == n_ and w_.is_contiguous()),
+             "qk_norm_pairs_store: norm weights")
+    if k is not None:
+        _chk(k.dim() == 4 and v.dim() == 4 and k.shape[1:] == (nkv, page_size, dk) and v.shape[1:] == (nkv, page_size, dv)
+             and k.shape[0] == v.shape[0] and k.is_contiguous() and v.is_contiguous() and k.dtype is v.dtype
+             and k.dtype in _DT and slot_map is not None, "qk_norm_pairs_store: cache")
+    if t:
+        _run("elementwise", "li_qk_norm_pairs_store", qkv.data_ptr(), qkv.stride(0), nh, nkv, dk, dv, rotary_dim,
+             0 if wq is None else wq.data_ptr(), 0 if wk is None else wk.data_ptr(), float(eps), cos.data_ptr(),
+             sin.data_ptr(), 0 if k is None else slot_map.data_ptr(), 0 if k is None else k.data_ptr(),
+             0 if k is None else v.data_ptr(), _DT[k.dtype] if k is not None else 0, page_size, int(k is not None), t)
+
+
+def latent_norm_pairs_store(qd: torch.Tensor, nh: int, dn: int, dr: int, rank: int, wc: torch.Tensor, eps: float,
+                            cos: torch.Tensor, sin: torch.Tensor, slot_map: Optional[torch.Tensor],
+                            cache: Optional[torch.Tensor], qfull: torch.Tensor) -> None:
+    """qd float32 rows [q (nh x (dn + dr)) | latent (rank) | shared rotated key part (dr)].  The latent is
+    RMS-normed and written with the rotated shared part to the token's page row [rank + dr]; every query head's
+    rotated part goes to columns rank.. of its row in qfull [T, nh, rank + dr] (float32)."""
+    _gpu(qd, wc, cos, sin, slot_map, cache, qfull)
+    t = qd.shape[0]
+    _chk(_rows_ok(qd) and qd.dtype is torch.float32 and qd.shape[1] >= nh * (dn + dr) + rank + dr,
+         "latent_norm_pairs_store: qd")
+    _chk(dr % 2 == 0 and dr > 0, "latent_norm_pairs_store: the rotated size must be even")
+    _check_tables("latent_norm_pairs_store", t, dr, cos, sin, slot_map if cache is not None else None)
+    _chk(wc.dtype is torch.float32 and wc.numel() == rank and wc.is_contiguous(), "latent_norm_pairs_store: norm weight")
+    _chk(qfull.shape == (t, nh, rank + dr) and qfull.is_contiguous() and qfull.dtype is torch.float32,
+         "latent_norm_pairs_store: qfull")
+    if cache is not None:
+        _chk(cache.dim() == 4 and cache.shape[1] == 1 and cache.shape[3] == rank + dr and cache.is_contiguous()
+             and cache.dtype in _DT and slot_map is not None, "latent_norm_pairs_store: cache [pages, 1, page, rank + dr]")
+    if t:
+        _run("elementwise", "li_latent_norm_pairs_store", qd.data_ptr(), qd.stride(0), nh, dn, dr, rank, wc.data_ptr(),
+             float(eps), cos.data_ptr(), sin.data_ptr(), 0 if cache is None else slot_map.data_ptr(),
+             0 if cache is None else cache.data_ptr(), _DT[cache.dtype] if cache is not None else 0, qfull.data_ptr(),
+             int(cache is not None), t)
+
+
+def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, out: torch.Tensor, k: torch.Tensor,
+                     v: torch.Tensor, meta, nh: int, nkv: int, dk: int, dv: int, page_size: int, window: int,
+                     keep_first: int, softcap: float, scale: float) -> None:
+    """Attention of every token of the step over its request's cached keys: position p sees j <= p with
+    p - j < window (0: all) or j < keep_first; scores (q . k) * scale, then softcap * tanh(score / softcap)
+    where softcap > 0; softmax and sums in float32.  q: a float32 tensor in which head h of token t starts at
+    t * q_token_stride + h * q_head_stride; k [pages, nkv, page, >= dk] and v [pages, nkv, page, >= dv] (the two
+    may be one tensor: then the value is the first dv columns of the key's row); out [T, nh * dv]."""
+    _gpu(q, out, k, v, meta.block_table)
+    t = out.shape[0]
+    _chk(q.dtype is torch.float32 and q.is_contiguous() and q.numel() >= (t - 1) * q_token_stride + (nh - 1) * q_head_stride + dk,
+         "masked_attention: q")
+    _chk(out.shape == (t, nh * dv) and out.is_contiguous() and out.dtype in _DT, "masked_attention: out")
+    _chk(k.dim() == 4 and v.dim() == 4 and k.shape[:3] == (k.shape[0], nkv, page_size) and v.shape[:3] == k.shape[:3]
+         and k.shape[3] >= dk and v.shape[3] >= dv and k.is_contiguous() and v.is_contiguous() and k.dtype is v.dtype
+         and k.dtype in _DT and (out.dtype is k.dtype or out.dtype is torch.float32), "masked_attention: cache")
+    _chk(nh % nkv == 0 and meta.num_tokens == t and meta.block_table.shape == (meta.num_segments, meta.max_blocks),
+         "masked_attention: batch")
+    if t:
+        _run("attention_masked", "li_masked_attention", q.data_ptr(), int(q_token_stride), int(q_head_stride),
+             out.data_ptr(), _DT[out.dtype], k.data_ptr(), v.data_ptr(), _DT[k.dtype], k.shape[3], v.shape[3],
+             meta.block_table.data_ptr(), meta.max_blocks, meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(),
+             meta.q_len.data_ptr(), meta.ctx_len.data_ptr(), t, nh, nkv, dk, dv, page_size, k.shape[0], int(window),
+             int(keep_first), float(softcap or 0.0), float(scale))
+
+
+def headwise_linear(x: torch.Tensor, x_token_stride: int, x_head_stride: int, m: torch.Tensor, out: torch.Tensor,
+                    o_token_stride: int, o_head_stride: int, tokens: int) -> None:
+    """out[t, h, j] = sum_k m[h, j, k] * x[t, h, k] for m [heads, n_out, n_in]; head h of token t starts at
+    t * token_stride + h * head_stride in x (n_in values) and in out (n_out values)."""
+    _gpu(x, m, out)
+    nh, n_out, n_in = m.shape
+    _chk(m.is_contiguous() and m.dtype in _DT and x.dtype in _DT and out.dtype in _DT and x.is_contiguous()
+         and out.is_contiguous(), "headwise_linear: operands")
+    _chk(x.numel() >= (tokens - 1) * x_token_stride + (nh - 1) * x_head_stride + n_in
+         and out.numel() >= (tokens - 1) * o_token_stride + (nh - 1) * o_head_stride + n_out
+         and x_head_stride >= 0 and o_head_stride >= n_out, "headwise_linear: strides")
+    _chk(m.dtype is torch.bfloat16 or (x.dtype is torch.float32 and out.dtype is torch.float32), "headwise_linear: dtypes")
+    _chk(n_in <= 2048, "headwise_linear: at most 2048 inputs a head")
+    if tokens:
+        _run("attention_masked", "li_headwise_linear", x.data_ptr(), _DT[x.dtype], int(x_token_stride), int(x_head_stride),
+             m.data_ptr(), _DT[m.dtype], out.data_ptr(), _DT[out.dtype], int(o_token_stride), int(o_head_stride),
+             tokens, nh, n_out, n_in)
 
 
 # ---------------------------------------------------------------------- gemm

@@ -1,15 +1,19 @@
 from .base import (BatchNeeds, Block, FeedForward, Mixer, Norm, PagedKVNeed, PagedNeed, PagedTensor, Part,
                    Runtime, StateNeed, build_part, needs_of, register_part)
-from .position import Position, RopeNeox
+from .position import Position, RopeNeox, RopePairs
 from .linear import Linear
-from .stream import ResidualStream
+from .stream import BranchStream, ResidualStream
 from .norm import RMSNorm
 from .attention import GQAttention
-from .mlp import SwiGLUMLP
-from .block import PreNormBlock
+from .masked_attention import LatentAttention, MaskedAttention
+from .mlp import ReluSquaredMLP, SwiGLUMLP
+from .block import PreNormBlock, SandwichBlock
+from .token_side import TokenSideInput
+from .inject import LoopEntry
 from .embedding import LinearHead, TokenEmbedding
 
 __all__ = ["BatchNeeds", "Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "PagedNeed", "PagedTensor",
            "Part", "Runtime", "StateNeed", "needs_of",
            "build_part", "register_part", "Position", "RopeNeox", "Linear", "ResidualStream", "RMSNorm",
-           "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding"]
+           "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding", "RopePairs", "BranchStream",
+           "MaskedAttention", "LatentAttention", "ReluSquaredMLP", "SandwichBlock", "TokenSideInput", "LoopEntry"]

@@ -50,6 +50,14 @@ class Runtime:
     keep_stored_precision: bool = False
     # stored dtype -> number of matrices that were rounded to bfloat16 when they were bound
     rounded: Dict[str, int] = field(default_factory=dict, compare=False, hash=False)
+    # tensor name -> the bound tensor, for a tensor that several parts read (one table cut into a slice a layer)
+    shared: Dict[str, torch.Tensor] = field(default_factory=dict, compare=False, hash=False)
+
+    def shared_matrix(self, name: str, fetch: Callable[[], torch.Tensor]) -> torch.Tensor:
+        """`matrix(fetch())`, bound once however many parts ask for the tensor of this name."""
+        if name not in self.shared:
+            self.shared[name] = self.matrix(fetch())
+        return self.shared[name]
 
     def matrix(self, t: torch.Tensor) -> torch.Tensor:
         """A stored matrix as this runtime multiplies with it.  In 32-bit mode
@@ -86,10 +94,12 @@ class PagedTensor:
 class PagedNeed:
     """What a mixer keeps per token in pages: any number of named tensors of any shapes;
     `window` > 0 keeps only the last `window` positions visible (older pages are given
-    back).  Entries of the execution order with equal needs share a page group: one page
-    id and one block table per request serve all of them."""
+    back); with `keep_first` > 0 the first so many positions of a request stay visible
+    beside the window, and their pages stay.  Entries of the execution order with equal
+    needs share a page group: one page id and one block table per request serve all of them."""
     tensors: Tuple[PagedTensor, ...]
     window: int = 0
+    keep_first: int = 0
 
     def bytes_per_token(self, default_dtype: torch.dtype) -> int:
         total = 0

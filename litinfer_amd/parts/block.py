@@ -4,6 +4,8 @@ The residual stream x is float32; mixer and feed-forward add into it through
 the `ResidualStream` they are given."""
 from __future__ import annotations
 
+import torch
+
 from .base import Block, build_part, register_part
 
 
@@ -52,4 +54,71 @@ class PreNormBlock(Block):
         stream.next_norm = None
 
 
+class SandwichBlock(Block):
+    """A norm before AND behind each sublayer: x += norm1b(mixer(norm1(x))), then, if the layer has a
+    feed-forward, x += norm2b(ffn(norm2(x))), then, if it has one, the layer's token input
+    (`parts/token_side.py`).  A sublayer writes into a branch buffer; the kernel that norms and adds it
+    also leaves the norm through which the stream is read next, where that is known."""
+
+    def __init__(self, spec, rt, parts):
+        super().__init__(spec, rt)
+        self.norm1 = build_part("norm", parts["norm1"], rt)
+        self.mixer = build_part("mixer", parts["mixer"], rt)
+        self.norm1b = build_part("norm", parts["norm1b"], rt)
+        self.ffn = self.norm2 = self.norm2b = self.token_input = None
+        if parts.get("feed_forward") is not None:
+            self.norm2 = build_part("norm", parts["norm2"], rt)
+            self.ffn = build_part("feed_forward", parts["feed_forward"], rt)
+            self.norm2b = build_part("norm", parts["norm2b"], rt)
+        if parts.get("token_input") is not None:
+            self.token_input = build_part("token_input", parts["token_input"], rt)
+        self._all = tuple(p for p in (self.norm1, self.mixer, self.norm1b, self.norm2, self.ffn, self.norm2b,
+                                      self.token_input) if p is not None)
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._all)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def batch_needs(self):
+        needs = super().batch_needs()
+        for p in self._all:
+            needs = needs.merged(p.batch_needs())
+        return needs
+
+    def expected_params(self):
+        e = {}
+        for p in self._all:
+            e.update(p.expected_params())
+        return e
+
+    def load_params(self, get):
+        for p in self._all:
+            p.load_params(get)
+
+    def first_norm(self):
+        return self.norm1
+
+    def forward(self, stream, ctx, cache):
+        from .stream import BranchStream
+        after = stream.next_norm                   # the norm that reads the stream after this block
+        stream.next_norm = None
+        xn = stream.normed(self.norm1, ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype))
+        y = ctx.ws.buffer("block.branch", stream.shape, torch.float32)
+        branch = BranchStream(y, ctx.ws)
+        self.mixer.forward(xn, branch, ctx, cache)
+        last = self.ffn is None and self.token_input is None
+        stream.add_normed(self.norm1b, branch.result(), self.norm2 if self.ffn is not None else (after if last else None))
+        if self.ffn is not None:
+            xn = stream.normed(self.norm2, ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype))
+            branch = BranchStream(y, ctx.ws)
+            self.ffn.forward(xn, branch, ctx)
+            stream.add_normed(self.norm2b, branch.result(), after if self.token_input is None else None)
+        if self.token_input is not None:
+            self.token_input.forward(stream, ctx, after)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

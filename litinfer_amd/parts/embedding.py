@@ -25,13 +25,14 @@ class TokenEmbedding(Part):
         super().__init__(spec, rt)
         self.vocab = int(spec.args["vocab_size"])
         self.hidden = int(spec.args["hidden_size"])
+        self.param = self.prefix + str(spec.args.get("param", "weight"))
         self.table = None
 
     def expected_params(self):
-        return {self.prefix + "weight": ParamSpec((self.vocab, self.hidden))}
+        return {self.param: ParamSpec((self.vocab, self.hidden))}
 
     def load_params(self, get):
-        self.table = self.rt.matrix(get(self.prefix + "weight"))
+        self.table = self.rt.matrix(get(self.param))
 
     def forward(self, ids, out, id_src=None, feedback=None):
         ops.embedding(ids, self.table, out, id_src, feedback)
@@ -50,21 +51,22 @@ class LinearHead(Part):
         self.tied_to = spec.args.get("tied_to")
         # untied by the configuration, but no matrix stored: use the table, as the reference does
         self.tie_if_absent = bool(spec.args.get("tie_if_absent", False))
+        self.param = self.prefix + str(spec.args.get("param", "weight"))
         self.proj = None
 
     def expected_params(self):
         if self.tied_to:
             return {}
-        return {self.prefix + "weight": ParamSpec((self.vocab, self.hidden), required=not self.tie_if_absent)}
+        return {self.param: ParamSpec((self.vocab, self.hidden), required=not self.tie_if_absent)}
 
     def load_params(self, get, tied_table=None):
         """`tied_table` is the embedding's table as the model holds it."""
-        w = None if self.tied_to else get(self.prefix + "weight")
+        w = None if self.tied_to else get(self.param)
         if w is None:
             if tied_table is None:
                 raise ValueError("head: tied to the embedding, but no table was given")
             if not self.tied_to and hasattr(get, "note"):
-                get.note(f"{self.prefix}weight is not stored: the head uses the embedding table")
+                get.note(f"{self.param} is not stored: the head uses the embedding table")
             self.proj = Linear(self.rt, tied_table)
         else:
             self.proj = Linear(self.rt, w)

@@ -1,0 +1,184 @@
+"""Two attention mixers over the paged cache that share one attention kernel (`ops.masked_attention`):
+a window beside which a number of first positions stay visible, scores capped by a tanh, keys and
+values of unequal sizes.
+
+`MaskedAttention`: grouped-query attention.  q = xn Wq^T, k = xn Wk^T, v = xn Wv^T (one packed
+product, left in float32); optionally an RMS norm over the WHOLE of q and the whole of k (all heads
+at once, before the split into heads); the position encoding on the first columns of every query and
+key head; score = (q . k) * scale, then cap * tanh(score / cap) where a cap is given; the query at
+position p sees the keys j <= p with p - j < window (0: all) or j < keep_first; softmax; Wo on the
+heads side by side.
+
+`LatentAttention`: keys and values are expanded from one latent vector c per token, c = the RMS
+norm of the first `rank` rows of Wd xn; the other `rot_dim` rows of Wd xn, rotated, are a key part
+that all heads share.  Head h has key [Wuk_h c | shared part] and value Wuv_h c, and a query of
+`dim` plain and `rot_dim` rotated columns.  Only c and the shared part are cached.  The expansion is
+never carried out per key: q_h . (Wuk_h c) = (Wuk_h^T q_h) . c, and sum_j p_j Wuv_h c_j =
+Wuv_h (sum_j p_j c_j), so the attention runs over the cached rows themselves, one kv head of
+rank + rot_dim key columns whose first `rank` are also the value, with a per-head product before
+(queries into the latent space) and one after it (the summed latent into the head's value space).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import ParamSpec
+from .base import BatchNeeds, Mixer, PagedNeed, PagedTensor, build_part, register_part
+from .linear import Linear
+
+
+class MaskedAttention(Mixer):
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        a = spec.args
+        self.hidden = int(a["hidden_size"])
+        self.nh = int(a["num_heads"])
+        self.nkv = int(a.get("num_kv_heads") or self.nh)
+        self.dk = int(a["head_dim"])
+        self.dv = int(a.get("value_dim") or self.dk)
+        self.window = int(a.get("window") or 0)
+        self.keep_first = int(a.get("keep_first") or 0) if self.window else 0
+        self.softcap = float(a.get("softcap") or 0.0)
+        self.scale = float(a["scale"]) if a.get("scale") is not None else self.dk ** -0.5
+        self.qk_norm = bool(a.get("qk_norm", False))
+        self.eps = float(a.get("eps", 1e-6))
+        if self.nh <= 0 or self.nkv <= 0 or self.nh % self.nkv:
+            raise ValueError(f"attention: {self.nh} heads are not a multiple of {self.nkv} kv heads")
+        if self.softcap < 0 or self.window < 0 or self.keep_first < 0:
+            raise ValueError("attention: the cap, the window and the kept first positions must not be negative")
+        self.position = build_part("position", a["position"], rt) if a.get("position") else None
+        self.rotary_dim = int(getattr(self.position, "rotary_dim", 0)) if self.position is not None else 0
+        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "q_norm": "q.norm", "k_norm": "k.norm",
+                      **(a.get("names") or {})}
+        self.n_q, self.n_k, self.n_v = self.nh * self.dk, self.nkv * self.dk, self.nkv * self.dv
+        self.qkv = self.out = self.wq = self.wk = None
+
+    @property
+    def graph_safe(self):
+        return self.position is None or self.position.graph_safe
+
+    def cache_need(self):
+        return PagedNeed((PagedTensor("k", (self.nkv, self.dk)), PagedTensor("v", (self.nkv, self.dv))),
+                         self.window, self.keep_first)
+
+    def batch_needs(self):
+        return BatchNeeds(row_tile=self.qkv.row_tile() if self.qkv is not None else 1)
+
+    def expected_params(self):
+        p, n = self.prefix, self.names
+        e = {p + n["q"]: ParamSpec((self.n_q, self.hidden)), p + n["k"]: ParamSpec((self.n_k, self.hidden)),
+             p + n["v"]: ParamSpec((self.n_v, self.hidden)), p + n["o"]: ParamSpec((self.hidden, self.nh * self.dv))}
+        if self.qk_norm:
+            e[p + n["q_norm"]] = ParamSpec((self.n_q,), init="one_plus_normal")
+            e[p + n["k_norm"]] = ParamSpec((self.n_k,), init="one_plus_normal")
+        return e
+
+    def load_params(self, get):
+        p, n = self.prefix, self.names
+        ws = [get(p + n[x]) for x in "qkv"]
+        dt = torch.float32 if any(w.dtype is torch.float32 for w in ws) else ws[0].dtype
+        self.qkv = Linear(self.rt, torch.cat([w.to(dt) for w in ws], dim=0))
+        self.out = Linear(self.rt, get(p + n["o"]))
+        if self.qk_norm:
+            self.wq, self.wk = self.rt.vector(get(p + n["q_norm"])), self.rt.vector(get(p + n["k_norm"]))
+
+    def forward(self, xn, residual, ctx, cache):
+        t = xn.shape[0]
+        qkv = ctx.ws.buffer("attn.qkv32", (t, self.n_q + self.n_k + self.n_v), torch.float32)
+        self.qkv(xn, qkv, ws=ctx.ws)
+        if self.position is not None:
+            cos, sin = self.position.tables(ctx)
+        else:
+            cos = sin = ctx.ws.buffer("attn.no_tables", (t, 0), torch.float32)
+        # norm over the whole projections, rotation, and the write of keys and values to their pages: one kernel
+        ops.qk_norm_pairs_store(qkv, self.nh, self.nkv, self.dk, self.dv, self.rotary_dim, self.wq, self.wk, self.eps,
+                                cos, sin, ctx.slot_map(cache.group) if cache.owned else None,
+                                cache.k if cache.owned else None, cache.v if cache.owned else None, cache.page_size)
+        attn = ctx.ws.buffer("attn.out", (t, self.nh * self.dv), self.rt.dtype)
+        ops.masked_attention(qkv, qkv.stride(0), self.dk, attn, cache.k, cache.v, ctx.attention_meta(cache.group),
+                             self.nh, self.nkv, self.dk, self.dv, cache.page_size, self.window, self.keep_first,
+                             self.softcap, self.scale)
+        residual.add_linear(self.out, attn)
+
+
+class LatentAttention(Mixer):
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        a = spec.args
+        self.hidden = int(a["hidden_size"])
+        self.nh = int(a["num_heads"])
+        self.dn = int(a["head_dim"])                 # plain (unrotated) query/key columns of a head
+        self.dr = int(a["rot_dim"])                  # rotated columns
+        self.dv = int(a.get("value_dim") or self.dn)
+        self.rank = int(a["kv_rank"])
+        self.window = int(a.get("window") or 0)
+        self.keep_first = int(a.get("keep_first") or 0) if self.window else 0
+        self.softcap = float(a.get("softcap") or 0.0)
+        self.scale = float(a["scale"]) if a.get("scale") is not None else (self.dn + self.dr) ** -0.5
+        self.eps = float(a.get("eps", 1e-6))
+        if min(self.nh, self.dn, self.dv, self.rank) <= 0 or self.dr <= 0 or self.dr % 2:
+            raise ValueError("latent attention: sizes must be positive and the rotated size even")
+        self.position = build_part("position", a["position"], rt)
+        if int(getattr(self.position, "rotary_dim", self.dr)) != self.dr:
+            raise ValueError("latent attention: the position encoding must rotate the whole rotated part")
+        self.names = {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_k": "uk", "up_v": "uv", "o": "o",
+                      **(a.get("names") or {})}
+        self.n_q = self.nh * (self.dn + self.dr)
+        self.q_down = self.out = self.wc = self.to_latent = self.from_latent = None
+
+    @property
+    def graph_safe(self):
+        return self.position.graph_safe
+
+    def cache_need(self):
+        # one row a token: the latent, then the shared rotated key part
+        return PagedNeed((PagedTensor("latent", (1, self.rank + self.dr)),), self.window, self.keep_first)
+
+    def batch_needs(self):
+        return BatchNeeds(row_tile=self.q_down.row_tile() if self.q_down is not None else 1)
+
+    def expected_params(self):
+        p, n = self.prefix, self.names
+        return {p + n["q"]: ParamSpec((self.n_q, self.hidden)),
+                p + n["down"]: ParamSpec((self.rank + self.dr, self.hidden)),
+                p + n["down_norm"]: ParamSpec((self.rank,), init="one_plus_normal"),
+                p + n["up_k"]: ParamSpec((self.nh * self.dn, self.rank)),
+                p + n["up_v"]: ParamSpec((self.nh * self.dv, self.rank)),
+                p + n["o"]: ParamSpec((self.hidden, self.nh * self.dv))}
+
+    def load_params(self, get):
+        p, n = self.prefix, self.names
+        wq, wd = get(p + n["q"]), get(p + n["down"])
+        dt = torch.float32 if torch.float32 in (wq.dtype, wd.dtype) else wq.dtype
+        self.q_down = Linear(self.rt, torch.cat([wq.to(dt), wd.to(dt)], dim=0))
+        self.wc = self.rt.vector(get(p + n["down_norm"]))
+        # per head: queries into the latent space (Wuk_h^T, [rank, dn]) and the summed latent out of it (Wuv_h, [dv, rank])
+        uk = get(p + n["up_k"]).reshape(self.nh, self.dn, self.rank).transpose(1, 2).contiguous()
+        self.to_latent = self.rt.matrix(uk)
+        self.from_latent = self.rt.matrix(get(p + n["up_v"]).reshape(self.nh, self.dv, self.rank).contiguous())
+        self.out = Linear(self.rt, get(p + n["o"]))
+
+    def forward(self, xn, residual, ctx, cache):
+        t, nh, dn, dr, rank = xn.shape[0], self.nh, self.dn, self.dr, self.rank
+        qd = ctx.ws.buffer("latent.qd32", (t, self.n_q + rank + dr), torch.float32)
+        self.q_down(xn, qd, ws=ctx.ws)
+        cos, sin = self.position.tables(ctx)
+        rows = cache.tensors["latent"]
+        qfull = ctx.ws.buffer("latent.q", (t, nh, rank + dr), torch.float32)
+        ops.latent_norm_pairs_store(qd, nh, dn, dr, rank, self.wc, self.eps, cos, sin,
+                                    ctx.slot_map(cache.group) if cache.owned else None,
+                                    rows if cache.owned else None, qfull)
+        ops.headwise_linear(qd, qd.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t)
+        summed = ctx.ws.buffer("latent.summed", (t, nh * rank), torch.float32)
+        ops.masked_attention(qfull, nh * (rank + dr), rank + dr, summed, rows, rows, ctx.attention_meta(cache.group),
+                             nh, 1, rank + dr, rank, cache.page_size, self.window, self.keep_first, self.softcap, self.scale)
+        heads = ctx.ws.buffer("attn.out", (t, nh * self.dv), self.rt.dtype)
+        ops.headwise_linear(summed, nh * rank, rank, self.from_latent, heads, nh * self.dv, self.dv, t)
+        residual.add_linear(self.out, heads)
+
+
+register_part("mixer", "masked_attention", MaskedAttention)
+register_part("mixer", "latent_attention", LatentAttention)

@@ -61,3 +61,40 @@ class SwiGLUMLP(FeedForward):
 
 
 register_part("feed_forward", "swiglu_mlp", SwiGLUMLP)
+
+
+class ReluSquaredMLP(FeedForward):
+    """Dense feed-forward with a squared ReLU: y = max(xn Wu^T, 0)^2 Wd^T, no biases.  The first product is
+    left in float32 and the activation rounds once to the engine's dtype."""
+    graph_safe = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.hidden = int(spec.args["hidden_size"])
+        self.inter = int(spec.args["intermediate_size"])
+        self.names = {"up": "up", "down": "down", **(spec.args.get("names") or {})}
+        self.up = None
+        self.down = None
+
+    def expected_params(self):
+        p = self.prefix
+        return {p + self.names["up"]: ParamSpec((self.inter, self.hidden)),
+                p + self.names["down"]: ParamSpec((self.hidden, self.inter))}
+
+    def batch_needs(self):
+        return BatchNeeds(row_tile=self.down.row_tile() if self.down is not None else 1)
+
+    def load_params(self, get):
+        self.up = Linear(self.rt, get(self.prefix + self.names["up"]))
+        self.down = Linear(self.rt, get(self.prefix + self.names["down"]))
+
+    def forward(self, xn, residual, ctx):
+        t = xn.shape[0]
+        u = ctx.ws.buffer("mlp.up32", (t, self.inter), torch.float32)
+        self.up(xn, u, ws=ctx.ws)
+        h = ctx.ws.buffer("mlp.h", (t, self.inter), self.rt.dtype)
+        ops.relu_squared(u, h)
+        residual.add_linear(self.down, h)
+
+
+register_part("feed_forward", "relu2_mlp", ReluSquaredMLP)

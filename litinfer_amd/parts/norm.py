@@ -17,13 +17,14 @@ class RMSNorm(Norm):
         self.eps = float(spec.args["eps"])
         if self.eps < 0:
             raise ValueError(f"rmsnorm: eps must not be negative, found {self.eps}")
+        self.param = self.prefix + str(spec.args.get("param", "weight"))     # the tensor's name behind the prefix
         self.weight = None
 
     def expected_params(self):
-        return {self.prefix + "weight": ParamSpec((self.size,), init="one_plus_normal")}
+        return {self.param: ParamSpec((self.size,), init="one_plus_normal")}
 
     def load_params(self, get):
-        self.weight = self.rt.vector(get(self.prefix + "weight"))
+        self.weight = self.rt.vector(get(self.param))
 
     def forward(self, x, out):
         ops.rmsnorm(x, self.weight, self.eps, out)

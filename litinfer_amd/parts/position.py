@@ -107,3 +107,76 @@ class RopeNeox(Position):
 
 
 register_part("position", "rope_neox", RopeNeox)
+
+
+class RopePairs(Position):
+    """Rotary encoding of NEIGHBOURING pairs: on the first `rotary_dim` columns of a head, columns
+    (2i, 2i+1) at position p become (u cos a - v sin a, v cos a + u sin a) with a = p * f_i and
+    f_i = theta^(-2i / rotary_dim); the other columns pass.  Optional `scaling` (a dict with factor,
+    original, fast, slow) is the YaRN rule: with dim(t) = rotary_dim ln(original / (2 pi t)) /
+    (2 ln theta), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rotary_dim - 1) and
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the frequency is f_i / factor * ramp_i +
+    f_i (1 - ramp_i), and cos and sin are multiplied by 0.1 ln(factor) + 1.  The frequencies are
+    worked out once on the host (float64, rounded to float32); the angle, cos and sin are float32."""
+    graph_safe = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        a = spec.args
+        self.head_dim = int(a["head_dim"])
+        self.rotary_dim = int(a.get("rotary_dim", self.head_dim))
+        self.theta = float(a["theta"])
+        self.scaling = dict(a["scaling"]) if a.get("scaling") else None
+        if self.theta <= 0:
+            raise ValueError(f"rope: theta must be positive, found {self.theta}")
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
+            raise ValueError(f"rope: rotary_dim must be even and within the head size "
+                             f"{self.head_dim}, found {self.rotary_dim}")
+        freq, self.amplitude = pair_frequencies(self.rotary_dim, self.theta, self.scaling)
+        self._freq_host = freq
+        self._freq = None
+
+    def key(self):
+        sc = tuple(sorted(self.scaling.items())) if self.scaling else None
+        return ("rope_pairs", self.rotary_dim, self.theta, sc)
+
+    def tables(self, ctx):
+        def make():
+            import torch
+            if self._freq is None:
+                self._freq = torch.tensor(self._freq_host, dtype=torch.float32, device=self.rt.device)
+            name = f"rope_pairs.{hash(self.key()) & 0xffffffff:x}"
+            cos = ctx.ws.buffer(name + ".cos", (ctx.num_tokens, self.rotary_dim // 2), ops.float32)
+            sin = ctx.ws.buffer(name + ".sin", (ctx.num_tokens, self.rotary_dim // 2), ops.float32)
+            ops.rope_freq_table(ctx.positions, self._freq, self.amplitude, cos, sin)
+            return cos, sin
+        return ctx.shared(self.key(), make)
+
+    def apply(self, qkv, n_heads_total, head_dim, ctx):
+        cos, sin = self.tables(ctx)
+        ops.rope_pairs_apply(qkv, n_heads_total, head_dim, self.rotary_dim, cos, sin)
+
+
+def pair_frequencies(rotary_dim: int, theta: float, scaling=None):
+    """([f_0 .. f_{rotary_dim/2 - 1}], amplitude of cos and sin) as `RopePairs` describes them."""
+    import math
+    half = rotary_dim // 2
+    freq = [theta ** (-2.0 * i / rotary_dim) for i in range(half)]
+    if not scaling:
+        return freq, 1.0
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+    if factor <= 0 or original <= 0:
+        raise ValueError(f"rope scaling: factor and original must be positive, found {factor}, {original}")
+
+    def dim_of(turns: float) -> float:
+        return rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+    lo = max(math.floor(dim_of(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(dim_of(float(scaling["slow"]))), rotary_dim - 1)
+    out = []
+    for i, f in enumerate(freq):
+        ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        out.append(f / factor * ramp + f * (1.0 - ramp))
+    return out, 0.1 * math.log(factor) + 1.0
+
+
+register_part("position", "rope_pairs", RopePairs)

@@ -29,6 +29,7 @@ class ResidualStream:
         self.next_norm = None                 # the norm through which the stream is read next, if known
         self._scaled = None                   # (norm, ScaledRows) left by the last add_linear
         self._normed = None                   # (norm, its result) left by the last add_linear
+        self.ws_dtype = torch.bfloat16        # the dtype in which normed rows are handed to the parts (the model sets it)
 
     @property
     def shape(self):
@@ -67,3 +68,43 @@ class ResidualStream:
             return self._normed[1]
         norm.forward(self.x, out)
         return out
+
+    def add_normed(self, norm, y: torch.Tensor, next_norm=None) -> None:
+        """x += norm(y) for the output y [T, H] (float32) of a sublayer that is normed BEFORE it joins the
+        stream.  `next_norm`: the norm through which the stream is read next, if the caller knows it; the same
+        kernel then leaves that norm of the new sum, and `normed(next_norm, ...)` hands it out."""
+        from ..kernels import ops
+        scaling = norm.as_scaling()
+        if scaling is None:
+            raise NotImplementedError("add_normed: the norm behind a sublayer must be an RMS norm with weights")
+        self._scaled = self._normed = None
+        nxt = next_norm.as_scaling() if next_norm is not None else None
+        if nxt is None:
+            ops.rmsnorm_add(y, scaling.weight, scaling.eps, self.x)
+            return
+        rows = self.ws.buffer("stream.normed_rows", self.x.shape, self.ws_dtype)
+        ops.rmsnorm_add(y, scaling.weight, scaling.eps, self.x, nxt.weight, nxt.eps, rows)
+        self._normed = (next_norm, rows)
+
+
+class BranchStream(ResidualStream):
+    """What ONE sublayer puts out, for arrangements that treat it (norm it, gate it) before it joins the
+    residual stream: the mixer or feed-forward is handed this in the stream's place, and its first
+    `add_linear` writes instead of adding."""
+
+    def __init__(self, y: torch.Tensor, ws):
+        super().__init__(y, ws)
+        self._fresh = True
+
+    def tensor(self) -> torch.Tensor:
+        if self._fresh:
+            self.x.zero_()
+            self._fresh = False
+        return self.x
+
+    def add_linear(self, linear, h: torch.Tensor) -> None:
+        linear(h, self.x, accumulate=not self._fresh, ws=self.ws)
+        self._fresh = False
+
+    def result(self) -> torch.Tensor:
+        return self.tensor()
