@@ -69,18 +69,19 @@ def visible(i, j, size, keep_first=0):
     return j < keep_first
 
 
-def masked_softmax_attention(q, k, v, scale, size, keep_first=0, softcap=None):
-    """q [T, H, dk], k [T, H, dk], v [T, H, dv] (keys already expanded to the query heads)."""
-    T, H, _ = q.shape
-    out = np.zeros((T, H, v.shape[-1]))
+def masked_softmax_attention(q, k, v, scale, size, keep_first=0, softcap=None, q_pos=None, k_pos=None):
+    """q [Tq, H, dk], k [Tk, H, dk], v [Tk, H, dv] (keys already expanded to the query heads); positions
+    default to 0..T-1 on both sides.  Returns [Tq, H, dv]."""
+    Tq, H, _ = q.shape
+    q_pos = np.arange(Tq) if q_pos is None else np.asarray(q_pos)
+    k_pos = np.arange(k.shape[0]) if k_pos is None else np.asarray(k_pos)
+    see = np.array([[visible(int(i), int(j), size, keep_first) for j in k_pos] for i in q_pos])
+    out = np.zeros((Tq, H, v.shape[-1]))
     for h in range(H):
         s = (q[:, h] @ k[:, h].T) * scale
         if softcap:
             s = softcap * np.tanh(s / softcap)
-        for i in range(T):
-            for j in range(T):
-                if not visible(i, j, size, keep_first):
-                    s[i, j] = -np.inf
+        s = np.where(see, s, -np.inf)
         s = s - s.max(axis=1, keepdims=True)
         p = np.exp(s)
         p /= p.sum(axis=1, keepdims=True)
