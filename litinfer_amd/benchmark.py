@@ -712,6 +712,113 @@ def check_long_decode(eng, cfg, prompt, chunk) -> Dict[str, object]:
     return out
 
 
+# ------------------------------------------------- two designs at equal layer sizes
+DESIGN_SIZES = {          # width, heads, kv heads, head size, feed-forward width, latent rank, rotated size, token-input width
+    "1.5b": (1536, 12, 2, 128, 8960, 512, 64, 256),
+    "7b": (3584, 28, 4, 128, 18944, 512, 64, 256),
+}
+DESIGN_WINDOW = 1024
+
+
+def tovasun_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, object]:
+    """A Tovasun model at the layer sizes of a Qwen2 family member: latent attention and windowed grouped-query
+    attention in turn, layers 1..2 passed twice, a token input of 256 columns a layer."""
+    width, heads, kv, dim, ff, rank, rot, side = DESIGN_SIZES[size]
+    scale = (dim + rot) ** -0.5
+    latent = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": ff},
+              "mixer": {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": dim, "kv_rank": rank, "scale": scale,
+                        "mask": {"size": DESIGN_WINDOW},
+                        "rot": {"base": 10000.0, "dims": rot,
+                                "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    attn = {"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+            "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 30.0,
+                      "mask": {"size": DESIGN_WINDOW, "keep_first": 4}, "rot": {"base": 10000.0, "dims": dim // 2}}}
+    return {"architecture": "Tovasun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "layers": [latent if i % 2 == 0 else attn for i in range(layers)],
+            "loop": {"start": 1, "stop": 3, "times": 2} if layers >= 4 else None, "token_side": {"dim": side}}
+
+
+def compare_designs(a) -> Dict[str, object]:
+    """Prefill and decode throughput of Tovasun beside Qwen2 at the same width, heads, feed-forward width,
+    window and number of layer runs (random weights, random cache content)."""
+    import numpy as np
+    import torch
+    from .engine import Engine, StepEntry
+    dev, rng = "cuda:0", np.random.default_rng(0)
+    out: Dict[str, object] = {}
+    sizes = [a.shape] if a.shape in DESIGN_SIZES else list(DESIGN_SIZES)
+    batches = (1, a.batch, 64)
+    for size in sizes:
+        layers = a.layers or 6
+        tcfg = tovasun_config(size, layers)
+        runs = layers + (2 if tcfg["loop"] else 0)
+        width, heads, kv, dim, ff = DESIGN_SIZES[size][:5]
+        qcfg = dict(SHAPES[size], num_hidden_layers=runs, vocab_size=32000, use_sliding_window=True,
+                    sliding_window=DESIGN_WINDOW, max_window_layers=0, max_position_embeddings=8192)
+        res = {}
+        for name, cfg, vocab in (("tovasun", tcfg, tcfg["vocab"]), ("qwen2", qcfg, qcfg["vocab_size"])):
+            eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
+                                     num_pages=(64 * (DESIGN_WINDOW + 64) + 2 * PREFILL_TOKENS) // PAGE, max_seqs=65)
+            for g in eng.cache.groups:
+                for data in g.data.values():
+                    data.normal_(0, 0.5)
+            r: Dict[str, object] = {"weights_GB": round(eng.model.weight_bytes() / 1e9, 3), "layer_runs": runs}
+            prompt = rng.integers(0, vocab, PREFILL_TOKENS).tolist()
+            times = []
+            for i in range(4):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                logits = eng.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+                eng.finish(f"p{i}")
+            if not bool(torch.isfinite(logits).all()):
+                raise RuntimeError(f"bench: non-finite logits after the prompt ({name})")
+            r["prefill_tok_s"] = round(PREFILL_TOKENS / min(times[1:]), 1)
+            r["prefill_ms"] = round(min(times[1:]) * 1e3, 3)
+            for b in batches:
+                rids = [f"d{b}_{i}" for i in range(b)]
+                for rid in rids:                     # the cache "holds" a context longer than the window
+                    eng.cache.admit(rid)
+                    eng.cache.reserve(rid, 2 * DESIGN_WINDOW)
+                    eng.cache.commit(rid, 2 * DESIGN_WINDOW)
+                toks = rng.integers(0, vocab, b).tolist()
+
+                def one():
+                    return eng.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, toks)])
+                for _ in range(a.warmup):
+                    one()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                for _ in range(a.steps):
+                    logits = one()
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t
+                if not bool(torch.isfinite(logits).all()):
+                    raise RuntimeError(f"bench: non-finite logits in the decode loop ({name}, batch {b})")
+                r[f"decode_b{b}_tok_s"] = round(b * a.steps / dt, 1)
+                r[f"decode_b{b}_ms"] = round(dt / a.steps * 1e3, 4)
+                for rid in rids:
+                    eng.finish(rid)
+            res[name] = r
+            log(f"{size} {name}: {r}")
+            del eng
+            torch.cuda.empty_cache()
+        res["tovasun_over_qwen2"] = {k: round(res["tovasun"][k] / res["qwen2"][k], 3)
+                                     for k in res["qwen2"] if k.endswith("tok_s")}
+        out[size] = res
+    first = out[sizes[0]]
+    return {"metric": f"decode tok/s (Tovasun at the Qwen2-{sizes[0]} layer sizes, batch {a.batch}, window {DESIGN_WINDOW})",
+            "value": first["tovasun"][f"decode_b{a.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
+            "warmup": a.warmup, "ms_per_step": first["tovasun"][f"decode_b{a.batch}_ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": a.dtype,
+            "data": "synthetic: seeded random token ids, random weights N(0, 0.02), random cache content",
+            "config": {"model": "Tovasun beside Qwen2 at equal layer sizes", "global_batch": a.batch,
+                       "seq_len": 2 * DESIGN_WINDOW, "prefill_tokens": PREFILL_TOKENS, "page_size": PAGE,
+                       "parallelism": "none (1 GPU)"},
+            "designs": out}
+
+
 def main(argv: Optional[List[str]] = None) -> int:
     ap = argparse.ArgumentParser(prog="bench.py", description=__doc__.split("\n\n")[0])
     ap.add_argument("--gpus", type=int, default=1)
@@ -720,8 +827,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in `config`)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
-    ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep"])
-    ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="sweep: the member of the family whose layer sizes are taken")
+    ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep", "designs"])
+    ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
+                    help="sweep: the member of the family whose layer sizes are taken (7b); designs: 1.5b or 7b (both)")
     ap.add_argument("--page-order-seed", type=int, default=0,
                     help="headline: the cache's pages are handed out in a shuffled order, as a pool that has served requests "
                          "does (negative: in the order of their numbers; a request's keys then lie in one piece, and "
@@ -740,6 +848,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--chunk-size", type=int, default=1024)
     ap.add_argument("--prompt-len", type=int, default=30000, help="long: tokens of each prompt")
     a = ap.parse_args(argv)
+    if a.mode != "designs":
+        a.shape = a.shape or "7b"
     if a.gpus != 1:
         print(f"bench.py: this engine runs on ONE GPU; --gpus {a.gpus} is not supported", flush=True)
         return 2
@@ -753,6 +863,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     elif a.mode == "serving":
         a.requests = a.requests or 128
         out = serving(a)
+    elif a.mode == "designs":
+        a.steps, a.warmup = min(a.steps, 32), min(a.warmup, 4)
+        out = compare_designs(a)
     else:
         out = long_prompts(a)
     if "environment" not in out:
