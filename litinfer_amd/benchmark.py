@@ -714,8 +714,8 @@ def check_long_decode(eng, cfg, prompt, chunk) -> Dict[str, object]:
 
 # ------------------------------------------------- two designs at equal layer sizes
 DESIGN_SIZES = {          # width, heads, kv heads, head size, feed-forward width, latent rank, rotated size, token-input width
-    "1.5b": (1536, 12, 2, 128, 8960, 512, 64, 256),
-    "7b": (3584, 28, 4, 128, 18944, 512, 64, 256),
+    "1.5b": (1536, 12, 2, 128, 8960, 256, 64, 256),
+    "7b": (3584, 28, 4, 128, 18944, 256, 64, 256),
 }
 DESIGN_WINDOW = 1024
 

@@ -11,20 +11,33 @@
 // then lo .. p, with lo the window's lower edge.
 __device__ __forceinline__ int visible_key(int i, int n_first, int lo) { return i < n_first ? i : lo + (i - n_first); }
 
-// One wave per (token, query head).  A lane takes one key of a round of 64 for the scores (its row read in
-// 16-byte pieces where the rows allow it), then one value column (and every 64th after it) for the sums.
-template <typename T, typename TO, int NC, bool VEC>
-__global__ __launch_bounds__(64) void masked_attention_wave_kernel(
+// Orders a wave's own LDS writes before its own later LDS reads (other lanes' data included: a wave's LDS
+// instructions are carried out in the order of their issue), without the block's barrier.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// The general kernel (any sizes, both dtypes): a block of NW waves per (token, query head); wave w takes the
+// rounds w, w + NW, ... of 64 visible keys.  In a round a lane takes one key for the scores (its row read in
+// 16-byte pieces where the rows allow it), then one value column (and every 64th after it) for the sums.  The
+// waves' running (maximum, sum, sums of values) are joined through LDS in wave order.
+template <typename T, typename TO, int NC, bool VEC, int NW>
+__global__ __launch_bounds__(64 * NW) void masked_attention_wave_kernel(
     const float* __restrict__ q, int q_token_stride, int q_head_stride, TO* __restrict__ out,
     const T* __restrict__ kc, const T* __restrict__ vc, int k_row, int v_row,
-    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ seg_of_token,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_list,
+    const int* __restrict__ seg_of_token,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
     int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale) {
     extern __shared__ float smem[];
-    float* qs = smem;                        // [dk]
-    float* ps = smem + dk;                   // [64]
-    int* rowoff = (int*)(ps + LI_WAVE);      // [64]
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    float* qs = smem;                                        // [dk]
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    float* ps = smem + dk + w * 128;                         // [64] a wave
+    int* rowoff = (int*)(ps + LI_WAVE);                      // [64] a wave
+    float* join = smem + dk + NW * 128;                      // [NW][dv + 2]
+    const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, h = blockIdx.y;
     const int s = seg_of_token[t];
     const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
@@ -33,14 +46,14 @@ __global__ __launch_bounds__(64) void masked_attention_wave_kernel(
     const int kvh = h / (nh / nkv);
     const int* table = block_table + (size_t)s * max_blocks;
     const float* qrow = q + (size_t)t * q_token_stride + (size_t)h * q_head_stride;
-    for (int d = lane; d < dk; d += LI_WAVE) qs[d] = qrow[d];
+    for (int d = threadIdx.x; d < dk; d += 64 * NW) qs[d] = qrow[d];
     __syncthreads();
 
     float m = -INFINITY, l = 0.f;
     float acc[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) acc[c] = 0.f;
-    for (int i0 = 0; i0 < n_keys; i0 += LI_WAVE) {
+    for (int i0 = 64 * w; i0 < n_keys; i0 += 64 * NW) {
         const int i = i0 + lane;
         float sc = -INFINITY;
         int ro = -1;
@@ -80,10 +93,9 @@ __global__ __launch_bounds__(64) void masked_attention_wave_kernel(
         const float alpha = (l == 0.f) ? 0.f : expf(m - m_new);
         const float e = (ro >= 0) ? expf(sc - m_new) : 0.f;
         l = l * alpha + wave_sum(e);
-        __syncthreads();
-        ps[lane] = e;
+        ps[lane] = e;                            // (a wave's own LDS traffic is ordered: the reads below follow these writes)
         rowoff[lane] = ro;
-        __syncthreads();
+        wave_lds_sync();
         const int nk = (n_keys - i0 < LI_WAVE) ? n_keys - i0 : LI_WAVE;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
@@ -97,30 +109,60 @@ __global__ __launch_bounds__(64) void masked_attention_wave_kernel(
                 acc[c] = a;
             }
         }
+        wave_lds_sync();                         // (the next round's writes follow these reads)
         m = m_new;
     }
     TO* orow = out + ((size_t)t * nh + h) * dv;
+    if constexpr (NW == 1) {
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-        const int d = lane + c * LI_WAVE;
-        if (d < dv) store_from_float(orow + d, l != 0.f ? acc[c] / l : 0.f);
+        for (int c = 0; c < NC; ++c) {
+            const int d = lane + c * LI_WAVE;
+            if (d < dv) store_from_float(orow + d, l != 0.f ? acc[c] / l : 0.f);
+        }
+    } else {
+        float* mine = join + (size_t)w * (dv + 2);
+        if (lane == 0) { mine[dv] = m; mine[dv + 1] = l; }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int d = lane + c * LI_WAVE;
+            if (d < dv) mine[d] = acc[c];
+        }
+        __syncthreads();
+        float mm = -INFINITY;
+        for (int x = 0; x < NW; ++x) mm = fmaxf(mm, join[(size_t)x * (dv + 2) + dv]);
+        float ll = 0.f;
+        float f[NW];
+#pragma unroll
+        for (int x = 0; x < NW; ++x) {
+            const float mx = join[(size_t)x * (dv + 2) + dv], lx = join[(size_t)x * (dv + 2) + dv + 1];
+            f[x] = (lx == 0.f) ? 0.f : expf(mx - mm);
+            ll += lx * f[x];
+        }
+        for (int d = threadIdx.x; d < dv; d += 64 * NW) {
+            float a = 0.f;
+#pragma unroll
+            for (int x = 0; x < NW; ++x) a += join[(size_t)x * (dv + 2) + d] * f[x];
+            store_from_float(orow + d, ll != 0.f ? a / ll : 0.f);
+        }
     }
 }
 
 template <typename T, typename TO, int NC>
 static int launch_masked(const float* q, int qts, int qhs, void* out, const void* kc, const void* vc, int k_row, int v_row,
-                         const int* block_table, int max_blocks, const int* seg_of_token, const int* q_start, const int* q_len,
-                         const int* ctx_len, int T_, int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window,
-                         int keep_first, float softcap, float scale, hipStream_t stream) {
-    const dim3 grid(T_, nh);
-    const size_t lds = (size_t)(dk + 2 * LI_WAVE) * 4;
+                         const int* block_table, int max_blocks, const int* token_list, int n_tokens, const int* seg_of_token,
+                         const int* q_start, const int* q_len,
+                         const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window,
+                         int keep_first, float softcap, float scale, int waves, hipStream_t stream) {
+    const dim3 grid(n_tokens, nh);
     constexpr int E = 16 / sizeof(T);
     const bool vec = dk % E == 0 && k_row % E == 0 && ((uintptr_t)kc % 16) == 0;
-#define MA_GO(V)                                                                                                             \
-    masked_attention_wave_kernel<T, TO, NC, V><<<grid, 64, lds, stream>>>(                                                   \
-        q, qts, qhs, (TO*)out, (const T*)kc, (const T*)vc, k_row, v_row, block_table, max_blocks, seg_of_token, q_start,     \
-        q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window, keep_first, softcap, scale)
-    if (vec) MA_GO(true); else MA_GO(false);
+#define MA_GO(V, NW)                                                                                                         \
+    masked_attention_wave_kernel<T, TO, NC, V, NW><<<grid, 64 * NW, (size_t)(dk + NW * 128 + NW * (dv + 2)) * 4, stream>>>(  \
+        q, qts, qhs, (TO*)out, (const T*)kc, (const T*)vc, k_row, v_row, block_table, max_blocks, token_list, seg_of_token,  \
+        q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window, keep_first, softcap, scale)
+    if (waves >= 8) { if (vec) MA_GO(true, 8); else MA_GO(false, 8); }
+    else if (waves >= 4) { if (vec) MA_GO(true, 4); else MA_GO(false, 4); }
+    else { if (vec) MA_GO(true, 1); else MA_GO(false, 1); }
 #undef MA_GO
     return li_launch_status();
 }
@@ -128,18 +170,22 @@ static int launch_masked(const float* q, int qts, int qhs, void* out, const void
 // q float32: head h of token t at q + t * q_token_stride + h * q_head_stride (dk values).  out [T, nh, dv] of
 // out_dtype.  kc / vc: rows of k_row / v_row elements of cache_dtype, row (page * nkv + kv head) * page_size + place;
 // the key is the first dk and the value the first dv elements of its row (the two may be the same memory).
+// token_list (or null: tokens 0 .. n_tokens - 1): the tokens this call takes.  waves: 1, 4 or 8 waves share a
+// (token, head)'s keys.
 extern "C" int li_masked_attention(const float* q, int q_token_stride, int q_head_stride, void* out, int out_dtype,
                                    const void* kc, const void* vc, int cache_dtype, int k_row, int v_row,
-                                   const int* block_table, int max_blocks, const int* seg_of_token, const int* q_start,
-                                   const int* q_len, const int* ctx_len, int T_, int nh, int nkv, int dk, int dv,
+                                   const int* block_table, int max_blocks, const int* token_list, int n_tokens,
+                                   const int* seg_of_token, const int* q_start,
+                                   const int* q_len, const int* ctx_len, int nh, int nkv, int dk, int dv,
                                    int page_size, int num_pages, int window, int keep_first, float softcap, float scale,
-                                   hipStream_t stream) {
-    if (T_ <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dv <= 0 || dk > k_row || dv > v_row || page_size <= 0 ||
-        window < 0 || keep_first < 0 || max_blocks <= 0 || nh > 65535 || dk > 8192 || dv > 64 * MA_MAX_CHUNKS)
+                                   int waves, hipStream_t stream) {
+    if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dk <= 0 || dv <= 0 || dk > k_row || dv > v_row || page_size <= 0 ||
+        window < 0 || keep_first < 0 || max_blocks <= 0 || nh > 65535 || dk > 4096 || dv > 64 * MA_MAX_CHUNKS)
         return LI_ERR_SIZE;
     const int nc = (dv + 63) / 64;
-#define MA_ARGS q, q_token_stride, q_head_stride, out, kc, vc, k_row, v_row, block_table, max_blocks, seg_of_token, q_start, \
-                q_len, ctx_len, T_, nh, nkv, dk, dv, page_size, num_pages, window, keep_first, softcap, scale, stream
+#define MA_ARGS q, q_token_stride, q_head_stride, out, kc, vc, k_row, v_row, block_table, max_blocks, token_list, n_tokens,  \
+                seg_of_token, q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window, keep_first, softcap,   \
+                scale, waves, stream
 #define MA_PICK(T, TO)                                                                  \
     {                                                                                   \
         if (nc <= 1) return launch_masked<T, TO, 1>(MA_ARGS);                           \
@@ -154,6 +200,201 @@ extern "C" int li_masked_attention(const float* q, int q_token_stride, int q_hea
 #undef MA_PICK
 #undef MA_ARGS
     return LI_ERR_DTYPE;
+}
+
+// ------------------------------------------------------------------------------------------- tiles of queries, MFMA
+// Portions of prompts in bfloat16: a block takes a tile of up to 32 consecutive queries of one request and one kv
+// head; its (up to four) waves are query heads of that kv head and share every block of 32 keys and values, which
+// the block stages in LDS.  A wave works on the TRANSPOSED scores S^T[key, query] = K Q^T (v_mfma_f32_32x32x16_bf16;
+// row operand K from LDS, column operand Q in registers as bfloat16): a lane then holds 16 keys of ITS query
+// (register r: key 8 (r / 4) + 4 (l / 32) + r % 4), so scale, cap, mask and softmax are arithmetic inside a lane plus
+// one exchange with lane l ^ 32, and the probabilities, rounded to bfloat16, are the column operand of
+// O^T[d, query] = V^T P^T as they are.  Its row operand V^T wants, for one value column, the keys
+// {16 s + 4 h + i, 16 s + 8 + 4 h + i : i < 4} side by side: the values are written to LDS transposed and in that
+// order.  The visible keys of a tile are its kept first positions and the window of its first to its last query;
+// they are walked as one list (`visible_key`), 32 at a time.
+typedef __bf16 ma_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float ma_f32x16 __attribute__((ext_vector_type(16)));
+union ma_frag8 { uint4 raw; uint32_t w[4]; ma_bf16x8 v; };
+#define MT_WAVES 4
+#define MT_VS 40                    // row stride of the transposed values: 32 key places and a pad that spreads the banks
+
+template <int KS, int DT>           // KS = dk / 16, DT = dv / 32
+__global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
+    const float* __restrict__ q, int q_token_stride, int q_head_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, int k_row, int v_row,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
+    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale) {
+    constexpr int DK = KS * 16, DV = DT * 32, KROW = DK + 8;
+    constexpr int NT = MT_WAVES * 64;
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[32 * KROW];       // [key place][dimension]
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[DV * MT_VS];      // [value column][key place, permuted]
+    __shared__ int rows[32];                                              // the cache row of each key place, -1: none
+    const int tile = blockIdx.x, kvh = blockIdx.y;
+    const int s = tiles[4 * tile], t0 = tiles[4 * tile + 1], ntok = tiles[4 * tile + 2];
+    const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);             // position of the tile's first query
+    const int p_last = p0 + ntok - 1;
+    const int lo_min = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+    const int n_first = keep_first < lo_min ? keep_first : lo_min;
+    const int n_keys = n_first + (p_last - lo_min + 1);
+    const int* table = block_table + (size_t)s * max_blocks;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, ql = lane & 31, h = lane >> 5;
+    const int rep = nh / nkv;
+    const int hh = blockIdx.z * MT_WAVES + w;                             // this wave's head within the group
+    const bool active = hh < rep;
+    const int head = kvh * rep + (active ? hh : 0);
+    const int pq = p0 + ql;                                               // this lane's query (ql >= ntok: none)
+    const int lq = (window > 0) ? pq - window + 1 : 0;
+
+    ma_frag8 qf[KS];
+    {
+        const float* qrow = q + (size_t)(t0 + (ql < ntok ? ql : 0)) * q_token_stride + (size_t)head * q_head_stride;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) {
+            const float4 a = *reinterpret_cast<const float4*>(qrow + 16 * st + 8 * h);
+            const float4 b = *reinterpret_cast<const float4*>(qrow + 16 * st + 8 * h + 4);
+            qf[st].w[0] = pack2_bf16(a.x, a.y); qf[st].w[1] = pack2_bf16(a.z, a.w);
+            qf[st].w[2] = pack2_bf16(b.x, b.y); qf[st].w[3] = pack2_bf16(b.z, b.w);
+        }
+    }
+    ma_f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    for (int i0 = 0; i0 < n_keys; i0 += 32) {
+        __syncthreads();                                                  // the block before has been read
+        if (threadIdx.x < 32) {
+            const int i = i0 + threadIdx.x;
+            int ro = -1;
+            if (i < n_keys) {
+                const int key = visible_key(i, n_first, lo_min);
+                const int page = table[key / page_size];
+                if (page >= 0 && page < num_pages) ro = (page * nkv + kvh) * page_size + key % page_size;
+            }
+            rows[threadIdx.x] = ro;
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < 32 * (DK / 8); i += NT) {
+            const int kk = i / (DK / 8), c = i % (DK / 8), ro = rows[kk];
+            uint4 raw = {0u, 0u, 0u, 0u};
+            if (ro >= 0) raw = *reinterpret_cast<const uint4*>(kc + (size_t)ro * k_row + 8 * c);
+            *reinterpret_cast<uint4*>(&Ks[kk * KROW + 8 * c]) = raw;
+        }
+        for (int i = threadIdx.x; i < 32 * (DV / 8); i += NT) {
+            const int kk = i % 32, c = i / 32, ro = rows[kk];             // (neighbouring threads: neighbouring key places)
+            uint4 raw = {0u, 0u, 0u, 0u};
+            if (ro >= 0) raw = *reinterpret_cast<const uint4*>(vc + (size_t)ro * v_row + 8 * c);
+            const int k16 = kk & 15, rem = k16 & 7;
+            const int place = (kk & 16) + 8 * (rem >> 2) + 4 * (k16 >> 3) + (rem & 3);
+            const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                Vt[(8 * c + 2 * e) * MT_VS + place] = (uint16_t)(wv[e] & 0xffffu);
+                Vt[(8 * c + 2 * e + 1) * MT_VS + place] = (uint16_t)(wv[e] >> 16);
+            }
+        }
+        __syncthreads();
+        if (!active) continue;
+        // ---- S^T = K Q^T
+        ma_f32x16 sv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = 0.f;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) {
+            ma_frag8 kf;
+            kf.raw = *reinterpret_cast<const uint4*>(&Ks[ql * KROW + 16 * st + 8 * h]);
+            sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[st].v, sv, 0, 0, 0);
+        }
+        // ---- scale, cap, mask, softmax over the keys of this lane's query
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = i0 + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int key = visible_key(i, n_first, lo_min);
+            float sc = sv[r] * scale;
+            if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+            const bool see = i < n_keys && rows[8 * (r >> 2) + 4 * h + (r & 3)] >= 0 && key <= pq && (key >= lq || key < keep_first);
+            sv[r] = see ? sc : -INFINITY;
+            mx = fmaxf(mx, sv[r]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
+        const float mn = fmaxf(m, mx);
+        const float ms = (mn == -INFINITY) ? 0.f : mn;                    // a query may see no key of this block
+        const float alpha = (m == -INFINITY) ? 1.f : expf(m - ms);        // (m = -inf: nothing summed yet)
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { sv[r] = expf(sv[r] - ms); psum += sv[r]; }
+        l = l * alpha + psum;
+        m = mn;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
+        ma_frag8 pf[2];
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pf[st].w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                ma_frag8 vf;
+                vf.raw = *reinterpret_cast<const uint4*>(&Vt[(32 * dt + ql) * MT_VS + 16 * st + 8 * h]);
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
+            }
+    }
+    if (!active) return;
+    l += __shfl_xor(l, 32, LI_WAVE);
+    if (ql >= ntok) return;
+    const float inv = l != 0.f ? 1.0f / l : 0.f;
+    bf16_t* orow = out + ((size_t)(t0 + ql) * nh + head) * DV;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {           // registers 4 rg .. 4 rg + 3: value columns 32 dt + 8 rg + 4 h ..
+            uint32_t* dst = reinterpret_cast<uint32_t*>(orow + 32 * dt + 8 * rg + 4 * h);
+            dst[0] = pack2_bf16(acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv);
+            dst[1] = pack2_bf16(acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv);
+        }
+}
+
+// 1 if the tile kernel takes these sizes (bfloat16 cache and output)
+extern "C" int li_masked_attention_tiles_takes(int dk, int dv) {
+#define MT_HAS(K, V) if (dk == K && dv == V) return 1;
+    MT_HAS(64, 64) MT_HAS(128, 128) MT_HAS(128, 64) MT_HAS(64, 128) MT_HAS(96, 64) MT_HAS(160, 128) MT_HAS(192, 128)
+    MT_HAS(256, 256) MT_HAS(320, 256) MT_HAS(288, 256)
+#undef MT_HAS
+    return 0;
+}
+
+extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int q_head_stride, void* out, const void* kc,
+                                         const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
+                                         const int* tiles, int num_tiles, const int* q_start, const int* q_len,
+                                         const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages,
+                                         int window, int keep_first, float softcap, float scale, hipStream_t stream) {
+    if (num_tiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
+        window < 0 || keep_first < 0 || max_blocks <= 0 || k_row % 8 || v_row % 8 || q_token_stride % 4 || q_head_stride % 4 ||
+        ((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) % 16 || (uintptr_t)out % 8 || !li_masked_attention_tiles_takes(dk, dv))
+        return LI_ERR_SIZE;
+    const int rep = nh / nkv;
+    const dim3 grid(num_tiles, nkv, (rep + MT_WAVES - 1) / MT_WAVES);
+#define MT_GO(K, V)                                                                                                        \
+    if (dk == K && dv == V) {                                                                                              \
+        masked_attention_tile_kernel<K / 16, V / 32><<<grid, MT_WAVES * 64, 0, stream>>>(                                  \
+            q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
+            max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale); \
+        return li_launch_status();                                                                                         \
+    }
+    MT_GO(64, 64) MT_GO(128, 128) MT_GO(128, 64) MT_GO(64, 128) MT_GO(96, 64) MT_GO(160, 128) MT_GO(192, 128)
+    MT_GO(256, 256) MT_GO(320, 256) MT_GO(288, 256)
+#undef MT_GO
+    return LI_ERR_SIZE;
 }
 
 // ------------------------------------------------------------------------------------------- per-head products
@@ -213,10 +454,78 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
     }
 }
 
+// The same product on the matrix cores, for bfloat16 matrices with n_in a multiple of 16 and n_out a multiple of
+// 32: a wave takes 32 tokens and 32 outputs of one head and works on the transposed tile (outputs x tokens), so
+// that both operands are 16-byte pieces of rows as they lie in memory (a matrix row's k-values; a token's
+// inputs, rounded to bfloat16 if they are float32) and a lane ends with four consecutive outputs of its token.
+template <typename TX, typename TO>
+__global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
+    const TX* __restrict__ x, long x_token_stride, int x_head_stride, const bf16_t* __restrict__ m, TO* __restrict__ out,
+    long o_token_stride, int o_head_stride, int T_, int n_out, int n_in) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, ql = lane & 31, h2 = lane >> 5;
+    const int head = blockIdx.y, t0 = blockIdx.x * 32;
+    const int j0 = (blockIdx.z * 4 + w) * 32;
+    if (j0 >= n_out) return;
+    const int tok = t0 + ql < T_ ? t0 + ql : T_ - 1;
+    const TX* xrow = x + (size_t)tok * x_token_stride + (size_t)head * x_head_stride + 8 * h2;
+    const bf16_t* mrow = m + ((size_t)head * n_out + j0 + ql) * n_in + 8 * h2;
+    ma_f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int k = 0; k < n_in; k += 16) {
+        ma_frag8 a, b;
+        a.raw = *reinterpret_cast<const uint4*>(mrow + k);
+        if constexpr (sizeof(TX) == 2) {
+            b.raw = *reinterpret_cast<const uint4*>(xrow + k);
+        } else {
+            const float4 u = *reinterpret_cast<const float4*>(xrow + k);
+            const float4 v = *reinterpret_cast<const float4*>(xrow + k + 4);
+            b.w[0] = pack2_bf16(u.x, u.y); b.w[1] = pack2_bf16(u.z, u.w);
+            b.w[2] = pack2_bf16(v.x, v.y); b.w[3] = pack2_bf16(v.z, v.w);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
+    }
+    if (t0 + ql >= T_) return;
+    TO* orow = out + (size_t)(t0 + ql) * o_token_stride + (size_t)head * o_head_stride + j0;
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {               // registers 4 rg .. 4 rg + 3: outputs 8 rg + 4 h2 ..
+        TO* dst = orow + 8 * rg + 4 * h2;
+        if constexpr (sizeof(TO) == 2) {
+            uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
+            d2[0] = pack2_bf16(acc[4 * rg], acc[4 * rg + 1]);
+            d2[1] = pack2_bf16(acc[4 * rg + 2], acc[4 * rg + 3]);
+        } else {
+            *reinterpret_cast<float4*>(dst) = float4{acc[4 * rg], acc[4 * rg + 1], acc[4 * rg + 2], acc[4 * rg + 3]};
+        }
+    }
+}
+
+template <typename TX, typename TO>
+static bool headwise_mfma(const void* x, long xts, int xhs, const void* m, void* out, long ots, int ohs, int T_, int nh,
+                          int n_out, int n_in, hipStream_t stream) {
+    const int ex = 16 / (int)sizeof(TX) / 2 * 2, eo = 4;       // elements that the 16-byte (32-byte) loads and the stores must start on
+    if (T_ < 16 || n_in % 16 || n_out % 32 || xts % ex || xhs % ex || ots % eo || ohs % eo ||
+        (uintptr_t)x % 16 || (uintptr_t)m % 16 || (uintptr_t)out % 16)
+        return false;
+    const dim3 grid((T_ + 31) / 32, nh, (n_out + 127) / 128);
+    headwise_linear_mfma_kernel<TX, TO><<<grid, 256, 0, stream>>>((const TX*)x, xts, xhs, (const bf16_t*)m, (TO*)out, ots, ohs,
+                                                                  T_, n_out, n_in);
+    return true;
+}
+
 extern "C" int li_headwise_linear(const void* x, int x_dtype, long x_token_stride, int x_head_stride, const void* m, int m_dtype,
                                   void* out, int out_dtype, long o_token_stride, int o_head_stride, int T_, int nh, int n_out,
                                   int n_in, hipStream_t stream) {
     if (T_ <= 0 || nh <= 0 || nh > 65535 || n_out <= 0 || n_in <= 0 || n_in > 2048) return LI_ERR_SIZE;
+    // many tokens against bfloat16 matrices of even sizes: the matrix cores
+    if (m_dtype == LI_BF16) {
+        bool took = false;
+        if (x_dtype == LI_F32 && out_dtype == LI_F32) took = headwise_mfma<float, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
+        else if (x_dtype == LI_F32 && out_dtype == LI_BF16) took = headwise_mfma<float, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
+        else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) took = headwise_mfma<bf16_t, bf16_t>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
+        else if (x_dtype == LI_BF16 && out_dtype == LI_F32) took = headwise_mfma<bf16_t, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
+        if (took) return li_launch_status();
+    }
     const int zs = (n_out + 255) / 256;
     const dim3 grid((T_ + HL_TOK - 1) / HL_TOK, nh, zs < 64 ? zs : 64);
     const size_t lds = (size_t)HL_TOK * n_in * 4;

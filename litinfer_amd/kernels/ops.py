@@ -46,7 +46,8 @@ _SIGNATURES = {
         "li_latent_norm_pairs_store": [P, I, I, I, I, I, P, F, P, P, P, P, I, P, I, I],
     },
     "attention_masked": {
-        "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, I, F, F],
+        "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I],
+        "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F],
         "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I],
     },
     "gemm": {
@@ -498,12 +499,45 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
          and k.dtype in _DT and (out.dtype is k.dtype or out.dtype is torch.float32), "masked_attention: cache")
     _chk(nh % nkv == 0 and meta.num_tokens == t and meta.block_table.shape == (meta.num_segments, meta.max_blocks),
          "masked_attention: batch")
-    if t:
+    if not t:
+        return
+    # keys that one query may see, as far as the host knows without looking at the contexts (a recorded step
+    # must not depend on them): decides how many waves share a (token, head)'s keys in the general kernel
+    bound = window + keep_first if window else meta.max_blocks * page_size
+    waves = 8 if bound >= 512 else 4 if bound >= 128 else 1
+
+    def general(token_list, n):
         _run("attention_masked", "li_masked_attention", q.data_ptr(), int(q_token_stride), int(q_head_stride),
              out.data_ptr(), _DT[out.dtype], k.data_ptr(), v.data_ptr(), _DT[k.dtype], k.shape[3], v.shape[3],
-             meta.block_table.data_ptr(), meta.max_blocks, meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(),
-             meta.q_len.data_ptr(), meta.ctx_len.data_ptr(), t, nh, nkv, dk, dv, page_size, k.shape[0], int(window),
-             int(keep_first), float(softcap or 0.0), float(scale))
+             meta.block_table.data_ptr(), meta.max_blocks, 0 if token_list is None else token_list.data_ptr(), n,
+             meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
+             nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale), waves)
+
+    # portions of prompts in bfloat16, at the sizes it has: tiles of queries on the matrix cores
+    if (meta.tiles is not None and meta.num_tiles and meta.tile_rows == MASKED_TILE_ROWS and k.dtype is torch.bfloat16
+            and out.dtype is torch.bfloat16 and masked_tiles_take(dk, dv) and k.shape[3] % 8 == 0 and v.shape[3] % 8 == 0
+            and q_token_stride % 4 == 0 and q_head_stride % 4 == 0 and q.data_ptr() % 16 == 0):
+        _run("attention_masked", "li_masked_attention_tiles", q.data_ptr(), int(q_token_stride), int(q_head_stride),
+             out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3], meta.block_table.data_ptr(), meta.max_blocks,
+             meta.tiles.data_ptr(), meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
+             nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale))
+        if meta.num_single:
+            general(meta.single_tokens, meta.num_single)       # (a list is there: the batch has tokens of both kinds)
+        return
+    general(None, t)
+
+
+MASKED_TILE_ROWS = 32         # queries of one request that a block of the matrix-core kernel takes
+
+
+def masked_tiles_take(dk: int, dv: int) -> bool:
+    """Whether the matrix-core kernel for portions has these key and value sizes (bfloat16)."""
+    f = _fn_cache.get(("attention_masked", "li_masked_attention_tiles_takes"))
+    if f is None:
+        f = build.load("attention_masked").li_masked_attention_tiles_takes
+        f.argtypes, f.restype = [c_int, c_int], c_int
+        _fn_cache[("attention_masked", "li_masked_attention_tiles_takes")] = f
+    return bool(f(int(dk), int(dv)))
 
 
 def headwise_linear(x: torch.Tensor, x_token_stride: int, x_head_stride: int, m: torch.Tensor, out: torch.Tensor,

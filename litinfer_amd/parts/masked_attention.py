@@ -64,7 +64,9 @@ class MaskedAttention(Mixer):
                          self.window, self.keep_first)
 
     def batch_needs(self):
-        return BatchNeeds(row_tile=self.qkv.row_tile() if self.qkv is not None else 1)
+        # the kernels take single-token segments and the others (tiles of queries) apart
+        return BatchNeeds(tile_rows=ops.MASKED_TILE_ROWS, token_kinds=True,
+                          row_tile=self.qkv.row_tile() if self.qkv is not None else 1)
 
     def expected_params(self):
         p, n = self.prefix, self.names
@@ -138,7 +140,8 @@ class LatentAttention(Mixer):
         return PagedNeed((PagedTensor("latent", (1, self.rank + self.dr)),), self.window, self.keep_first)
 
     def batch_needs(self):
-        return BatchNeeds(row_tile=self.q_down.row_tile() if self.q_down is not None else 1)
+        return BatchNeeds(tile_rows=ops.MASKED_TILE_ROWS, token_kinds=True,
+                          row_tile=self.q_down.row_tile() if self.q_down is not None else 1)
 
     def expected_params(self):
         p, n = self.prefix, self.names
@@ -172,7 +175,7 @@ class LatentAttention(Mixer):
                                     ctx.slot_map(cache.group) if cache.owned else None,
                                     rows if cache.owned else None, qfull)
         ops.headwise_linear(qd, qd.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t)
-        summed = ctx.ws.buffer("latent.summed", (t, nh * rank), torch.float32)
+        summed = ctx.ws.buffer("latent.summed", (t, nh * rank), self.rt.dtype)
         ops.masked_attention(qfull, nh * (rank + dr), rank + dr, summed, rows, rows, ctx.attention_meta(cache.group),
                              nh, 1, rank + dr, rank, cache.page_size, self.window, self.keep_first, self.softcap, self.scale)
         heads = ctx.ws.buffer("attn.out", (t, nh * self.dv), self.rt.dtype)

@@ -196,10 +196,17 @@ def _meta(seg_specs, page, tables):
     q_start = np.concatenate([[0], np.cumsum(q_len)[:-1]]).astype(np.int32)
     seg_of = np.repeat(np.arange(len(seg_specs), dtype=np.int32), q_len)
     dev = lambda a: torch.from_numpy(a).to(DEV)
+    single = np.nonzero(q_len[seg_of] == 1)[0].astype(np.int32)
+    multi = np.nonzero(q_len[seg_of] != 1)[0].astype(np.int32)
+    tiles = np.asarray([(i, int(q_start[i]) + a, min(32, int(q_len[i]) - a), 0) for i in range(len(seg_specs))
+                        if q_len[i] > 1 for a in range(0, int(q_len[i]), 32)], dtype=np.int32).reshape(-1, 4)
     return AttentionMeta(block_table=dev(tables), max_blocks=tables.shape[1], seg_of_token=dev(seg_of),
                          q_start=dev(q_start), q_len=dev(q_len), ctx_len=dev(ctx_len), num_segments=len(seg_specs),
                          num_tokens=int(q_len.sum()), max_q_len=int(q_len.max()), max_ctx_len=int(ctx_len.max()),
-                         host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len)
+                         host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len,
+                         single_tokens=dev(single) if len(multi) else None, num_single=len(single),
+                         multi_tokens=dev(multi) if len(single) else None, num_multi=len(multi),
+                         tiles=dev(tiles), num_tiles=len(tiles), tile_rows=32)
 
 
 def _masked_case(dtype, seg_specs, nh, nkv, dk, dv, page, window, keep_first, softcap, seed, standout=None,
@@ -281,6 +288,12 @@ def _close(got, ref, dtype):
     ([(130, 130), (257, 3)], 4, 4, 128, 128, 32, 40, 4, 0.0),
     ([(500, 1), (90, 1), (3, 1), (41, 1)], 5, 5, 20, 12, 8, 40, 4, 7.5),         # decoding only
     ([(90, 30)], 3, 1, 300, 260, 16, 50, 2, 0.0),                      # long rows: several value columns a lane
+    # sizes that the matrix-core kernel for portions takes in bfloat16; single tokens beside the portions
+    ([(100, 37), (33, 2), (300, 1), (70, 70), (64, 64), (1, 1)], 6, 3, 64, 64, 8, 20, 5, 3.0),
+    ([(257, 100), (90, 90), (64, 33), (700, 1)], 10, 2, 128, 64, 16, 50, 0, 0.0),       # five heads a group: two turns of waves
+    ([(200, 130), (40, 40)], 7, 1, 96, 64, 16, 0, 0, 10.0),            # seven heads on one kv head, no window
+    ([(300, 200)], 4, 2, 64, 128, 32, 100, 33, 0.0),
+    ([(150, 150), (500, 35)], 3, 1, 320, 256, 16, 64, 1, 0.0),
 ])
 def test_masked_attention_against_the_plain_attention(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap):
     got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3)
@@ -291,11 +304,14 @@ def test_masked_attention_against_the_plain_attention(dtype, segs, nh, nkv, dk, 
 def test_values_that_are_the_first_columns_of_the_keys_rows(dtype):
     got, ref = _masked_case(dtype, [(120, 50), (77, 1)], 6, 1, 56, 40, 16, 30, 0, 0.0, seed=4, shared_rows=True)
     _close(got, ref, dtype)
+    got, ref = _masked_case(dtype, [(400, 70), (77, 1), (33, 33)], 6, 1, 160, 128, 16, 90, 0, 0.0, seed=5, shared_rows=True)
+    _close(got, ref, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("ql", [1, 40])
 @pytest.mark.parametrize("where", ["edge_in", "edge_out", "kept_in", "kept_out", "page_border", "self"])
-def test_one_standout_key_at_the_edges_of_window_and_kept_positions(where, ql):
+def test_one_standout_key_at_the_edges_of_window_and_kept_positions(where, ql, dtype):
     """Context 400, window 64, 3 kept positions, pages of 16.  One key is given a score that wins by e^12: just
     inside the window's edge it must dominate the output of the last query, just outside it must not; the same
     for the last kept position and the first one that is not kept."""
@@ -303,11 +319,11 @@ def test_one_standout_key_at_the_edges_of_window_and_kept_positions(where, ql):
     p = c - 1
     key = {"edge_in": p - window + 1, "edge_out": p - window, "kept_in": keep - 1, "kept_out": keep,
            "page_border": p - (p % page), "self": p}[where]
-    got, ref, values = _masked_case(torch.float32, [(c, ql)], 4, 2, 32, 32, page, window, keep, 0.0, seed=9,
+    got, ref, values = _masked_case(dtype, [(c, ql)], 4, 2, 64, 64, page, window, keep, 0.0, seed=9,
                                     standout=(key, None), return_values=True)
-    _close(got, ref, torch.float32)
+    _close(got, ref, dtype)
     # the last query's output is the standout key's value exactly when that key is visible
-    dominated = np.abs(got[-1].reshape(4, 32) - values[0][key]).max() < 0.05
+    dominated = np.abs(got[-1].reshape(4, 64) - values[0][key]).max() < 0.05
     assert dominated == (where not in ("edge_out", "kept_out"))
 
 
@@ -379,15 +395,17 @@ def test_squared_relu_gelu_gate_and_the_stream_additions():
 def test_products_with_a_matrix_of_its_own_for_every_head(dtype):
     from litinfer_amd.kernels import ops
     g = torch.Generator().manual_seed(4)
-    for t, nh, n_out, n_in, pad in ((1, 3, 40, 16, 8), (19, 5, 300, 72, 0), (64, 2, 24, 130, 6)):
+    # (the last three: sizes that go to the matrix cores in bfloat16, 32 tokens a tile)
+    for t, nh, n_out, n_in, pad, opad in ((1, 3, 40, 16, 8, 3), (19, 5, 300, 72, 0, 3), (64, 2, 24, 130, 6, 3),
+                                          (40, 3, 128, 64, 8, 4), (100, 4, 64, 160, 0, 0), (33, 2, 256, 48, 16, 8)):
         m = torch.randn(nh, n_out, n_in, generator=g).to(dtype)
         x = torch.randn(t, nh, n_in + pad, generator=g)              # a head's inputs lie inside a wider row
-        out = torch.zeros(t, nh, n_out + 3, dtype=dtype, device=DEV)
-        ops.headwise_linear(x.to(DEV), nh * (n_in + pad), n_in + pad, m.to(DEV), out, nh * (n_out + 3), n_out + 3, t)
+        out = torch.zeros(t, nh, n_out + opad, dtype=dtype, device=DEV)
+        ops.headwise_linear(x.to(DEV), nh * (n_in + pad), n_in + pad, m.to(DEV), out, nh * (n_out + opad), n_out + opad, t)
         ref = np.einsum("hjk,thk->thj", m.double().numpy(), x[..., :n_in].double().numpy())
         got = out.float().cpu().numpy()
         assert np.abs(got[..., :n_out] - ref).max() / np.abs(ref).max() < (1e-5 if dtype is torch.float32 else 1e-2)
-        assert np.abs(got[..., n_out:]).max() == 0                   # nothing written beside a head's outputs
+        assert opad == 0 or np.abs(got[..., n_out:]).max() == 0      # nothing written beside a head's outputs
 
 
 def test_mixers_alone_against_their_plain_forms(models):
