@@ -397,6 +397,234 @@ extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int
     return LI_ERR_SIZE;
 }
 
+// ------------------------------------------------------------------------------------------- single tokens, bfloat16
+// Decoding: one query a request, so the work is reading its visible keys and values once.  A block of four waves
+// takes one (token, kv head) and RH query heads of that kv head, so that a row is read once for all of them.  A
+// key's row is spread over 8 lanes, 16 bytes a lane and piece (lane j holds the pieces j, j + 8, ...): a wave takes
+// 8 keys at a time, the block 32, and U such rounds are in flight.  Every group of 8 lanes keeps a running
+// (maximum, sum, sums of values) per head over its keys; the groups of a wave are joined by a butterfly, the waves
+// through LDS in wave order.
+__device__ __forceinline__ void unpack8(const uint4 raw, float* f) {
+    f[0] = __uint_as_float(raw.x << 16); f[1] = __uint_as_float(raw.x & 0xffff0000u);
+    f[2] = __uint_as_float(raw.y << 16); f[3] = __uint_as_float(raw.y & 0xffff0000u);
+    f[4] = __uint_as_float(raw.z << 16); f[5] = __uint_as_float(raw.z & 0xffff0000u);
+    f[6] = __uint_as_float(raw.w << 16); f[7] = __uint_as_float(raw.w & 0xffff0000u);
+}
+
+template <int NPK, int NPV, int RH, int U>
+__global__ __launch_bounds__(256) void masked_attention_single_kernel(
+    const float* __restrict__ q, int q_token_stride, int q_head_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, int k_row, int v_row,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_list,
+    const int* __restrict__ seg_of_token, const int* __restrict__ q_start, const int* __restrict__ q_len,
+    const int* __restrict__ ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window,
+    int keep_first, float softcap, float scale) {
+    extern __shared__ float join[];                 // [4 waves][RH][dv + 2]
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, g = lane >> 3, j = lane & 7;
+    const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, kvh = blockIdx.y;
+    const int rep = nh / nkv, hfirst = blockIdx.z * RH;
+    const int nheads = rep - hfirst < RH ? rep - hfirst : RH;
+    const int s = seg_of_token[t];
+    const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int n_first = keep_first < lo ? keep_first : lo;
+    const int n_keys = n_first + (p - lo + 1);
+    const int* table = block_table + (size_t)s * max_blocks;
+
+    float qr[RH][NPK][8];
+#pragma unroll
+    for (int hh = 0; hh < RH; ++hh) {
+        const float* qrow = q + (size_t)t * q_token_stride + (size_t)(kvh * rep + hfirst + (hh < nheads ? hh : 0)) * q_head_stride;
+#pragma unroll
+        for (int c = 0; c < NPK; ++c) {
+            const int d0 = 8 * (j + 8 * c);
+            const bool on = d0 < dk && hh < nheads;
+            const float4 a = on ? *reinterpret_cast<const float4*>(qrow + d0) : float4{0.f, 0.f, 0.f, 0.f};
+            const float4 b = on ? *reinterpret_cast<const float4*>(qrow + d0 + 4) : float4{0.f, 0.f, 0.f, 0.f};
+            qr[hh][c][0] = a.x; qr[hh][c][1] = a.y; qr[hh][c][2] = a.z; qr[hh][c][3] = a.w;
+            qr[hh][c][4] = b.x; qr[hh][c][5] = b.y; qr[hh][c][6] = b.z; qr[hh][c][7] = b.w;
+        }
+    }
+    float acc[RH][NPV][8];
+    float m[RH], l[RH];
+#pragma unroll
+    for (int hh = 0; hh < RH; ++hh) {
+        m[hh] = -INFINITY; l[hh] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NPV; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[hh][c][e] = 0.f;
+    }
+    for (int i0 = 0; i0 < n_keys; i0 += 32 * U) {
+        size_t ro[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + 32 * u + 8 * w + g;
+            ok[u] = i < n_keys;
+            const int key = visible_key(ok[u] ? i : 0, n_first, lo);
+            const int page = table[key / page_size];
+            ok[u] = ok[u] && page >= 0 && page < num_pages;
+            ro[u] = ok[u] ? (size_t)(page * nkv + kvh) * page_size + key % page_size : 0;      // (row 0 exists: read, not used)
+        }
+        uint4 kp[U][NPK], vp[U][NPV];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int c = 0; c < NPK; ++c) {
+                const int d0 = 8 * (j + 8 * c);
+                kp[u][c] = *reinterpret_cast<const uint4*>(kc + ro[u] * k_row + (d0 < dk ? d0 : 0));
+            }
+#pragma unroll
+            for (int c = 0; c < NPV; ++c) {
+                const int d0 = 8 * (j + 8 * c);
+                vp[u][c] = *reinterpret_cast<const uint4*>(vc + ro[u] * v_row + (d0 < dv ? d0 : 0));
+            }
+        }
+        float sc[U][RH];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float kf[NPK][8];
+#pragma unroll
+            for (int c = 0; c < NPK; ++c) unpack8(kp[u][c], kf[c]);
+#pragma unroll
+            for (int hh = 0; hh < RH; ++hh) {
+                float d = 0.f;
+#pragma unroll
+                for (int c = 0; c < NPK; ++c)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) d = fmaf(qr[hh][c][e], kf[c][e], d);      // (pieces past dk meet zeros of q)
+                d += __shfl_xor(d, 1, LI_WAVE);
+                d += __shfl_xor(d, 2, LI_WAVE);
+                d += __shfl_xor(d, 4, LI_WAVE);
+                d *= scale;
+                if (softcap > 0.f) d = softcap * tanhf(d / softcap);
+                sc[u][hh] = ok[u] ? d : -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int hh = 0; hh < RH; ++hh) {
+            float mx = sc[0][hh];
+#pragma unroll
+            for (int u = 1; u < U; ++u) mx = fmaxf(mx, sc[u][hh]);
+            const float mn = fmaxf(m[hh], mx);
+            const float ms = (mn == -INFINITY) ? 0.f : mn;
+            const float alpha = (m[hh] == -INFINITY) ? 0.f : expf(m[hh] - ms);
+            float pu[U], psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < U; ++u) { pu[u] = expf(sc[u][hh] - ms); psum += pu[u]; }
+            l[hh] = l[hh] * alpha + psum;
+            m[hh] = mn;
+#pragma unroll
+            for (int c = 0; c < NPV; ++c) {
+                float a8[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a8[e] = acc[hh][c][e] * alpha;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    float vf[8];
+                    unpack8(vp[u][c], vf);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) a8[e] = fmaf(pu[u], vf[e], a8[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[hh][c][e] = a8[e];
+            }
+        }
+    }
+    // the groups of a wave
+#pragma unroll
+    for (int off = 8; off < 64; off <<= 1) {
+#pragma unroll
+        for (int hh = 0; hh < RH; ++hh) {
+            const float m2 = __shfl_xor(m[hh], off, LI_WAVE), l2 = __shfl_xor(l[hh], off, LI_WAVE);
+            const float mn = fmaxf(m[hh], m2);
+            const float f1 = (m[hh] == -INFINITY) ? 0.f : expf(m[hh] - mn), f2 = (m2 == -INFINITY) ? 0.f : expf(m2 - mn);
+            l[hh] = l[hh] * f1 + l2 * f2;
+            m[hh] = mn;
+#pragma unroll
+            for (int c = 0; c < NPV; ++c)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[hh][c][e] = acc[hh][c][e] * f1 + __shfl_xor(acc[hh][c][e], off, LI_WAVE) * f2;
+        }
+    }
+    // the waves
+    if (g == 0) {
+#pragma unroll
+        for (int hh = 0; hh < RH; ++hh) {
+            float* mine = join + (size_t)(w * RH + hh) * (dv + 2);
+            if (j == 0) { mine[dv] = m[hh]; mine[dv + 1] = l[hh]; }
+#pragma unroll
+            for (int c = 0; c < NPV; ++c) {
+                const int d0 = 8 * (j + 8 * c);
+                if (d0 < dv)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) mine[d0 + e] = acc[hh][c][e];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nheads * dv; idx += 256) {
+        const int hh = idx / dv, d = idx % dv;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) mm = fmaxf(mm, join[(size_t)(x * RH + hh) * (dv + 2) + dv]);
+        float a = 0.f, ll = 0.f;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const float* r = join + (size_t)(x * RH + hh) * (dv + 2);
+            const float f = (r[dv] == -INFINITY) ? 0.f : expf(r[dv] - mm);
+            a += r[d] * f;
+            ll += r[dv + 1] * f;
+        }
+        out[((size_t)t * nh + kvh * rep + hfirst + hh) * dv + d].bits = float_to_bf16(ll != 0.f ? a / ll : 0.f);
+    }
+}
+
+// 1 if the kernel for single tokens takes these sizes (bfloat16 cache and output)
+extern "C" int li_masked_attention_single_takes(int dk, int dv) {
+    const int npk = (dk + 63) / 64, npv = (dv + 63) / 64;
+    if (dk % 8 || dv % 8 || dk <= 0 || dv <= 0) return 0;
+    return (npk <= 2 && npv <= 2) || (npk == 3 && npv == 2) || (npk == 4 && npv == 4) || (npk == 5 && npv == 4) || (npk == 4 && npv == 3);
+}
+
+extern "C" int li_masked_attention_single(const float* q, int q_token_stride, int q_head_stride, void* out, const void* kc,
+                                          const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
+                                          const int* token_list, int n_tokens, const int* seg_of_token, const int* q_start,
+                                          const int* q_len, const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size,
+                                          int num_pages, int window, int keep_first, float softcap, float scale,
+                                          hipStream_t stream) {
+    if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
+        window < 0 || keep_first < 0 || max_blocks <= 0 || num_pages <= 0 || k_row % 8 || v_row % 8 || q_token_stride % 4 ||
+        q_head_stride % 4 || ((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) % 16 || !li_masked_attention_single_takes(dk, dv))
+        return LI_ERR_SIZE;
+    const int rep = nh / nkv, npk = (dk + 63) / 64, npv = (dv + 63) / 64;
+    const int rh = (npk + npv > 6) ? (rep >= 2 ? 2 : 1) : (rep >= 4 && (rep % 4 == 0 || rep % 4 == 3 || rep > 8)) ? 4 : rep >= 2 ? 2 : 1;
+    const dim3 grid(n_tokens, nkv, (rep + rh - 1) / rh);
+    const size_t lds = (size_t)4 * rh * (dv + 2) * 4;
+#define MS_GO(K, V, R, UU)                                                                                                  \
+    masked_attention_single_kernel<K, V, R, UU><<<grid, 256, lds, stream>>>(                                                \
+        q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table,    \
+        max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window,       \
+        keep_first, softcap, scale)
+#define MS_SMALL(K, V)                                                                                                      \
+    if (npk == K && npv == V) {                                                                                             \
+        if (rh == 4) MS_GO(K, V, 4, 4); else if (rh == 2) MS_GO(K, V, 2, 4); else MS_GO(K, V, 1, 4);                        \
+        return li_launch_status();                                                                                          \
+    }
+#define MS_LARGE(K, V)                                                                                                      \
+    if (npk == K && npv == V) {                                                                                             \
+        if (rh == 2) MS_GO(K, V, 2, 2); else MS_GO(K, V, 1, 2);                                                             \
+        return li_launch_status();                                                                                          \
+    }
+    MS_SMALL(1, 1) MS_SMALL(2, 1) MS_SMALL(1, 2) MS_SMALL(2, 2) MS_SMALL(3, 2)
+    MS_LARGE(4, 4) MS_LARGE(5, 4) MS_LARGE(4, 3)
+#undef MS_GO
+#undef MS_SMALL
+#undef MS_LARGE
+    return LI_ERR_SIZE;
+}
+
 // ------------------------------------------------------------------------------------------- per-head products
 // out[t, h, j] = sum_k m[h, j, k] * x[t, h, k]: every head has a matrix of its own, [n_out, n_in], stored one after
 // the other.  x and out are addressed by a token stride and a head stride, so that a head's columns may lie inside

@@ -47,6 +47,7 @@ _SIGNATURES = {
     },
     "attention_masked": {
         "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I],
+        "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F],
         "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F],
         "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I],
     },
@@ -513,21 +514,45 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
              meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale), waves)
 
+    fast = (k.dtype is torch.bfloat16 and out.dtype is torch.bfloat16 and k.shape[3] % 8 == 0 and v.shape[3] % 8 == 0
+            and q_token_stride % 4 == 0 and q_head_stride % 4 == 0 and q.data_ptr() % 16 == 0)
+
+    def singles(token_list, n):
+        # single tokens in bfloat16, at the sizes it has: rows spread over lanes, a row read once for a group's heads
+        if not (fast and masked_single_takes(dk, dv)):
+            return general(token_list, n)
+        _run("attention_masked", "li_masked_attention_single", q.data_ptr(), int(q_token_stride), int(q_head_stride),
+             out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3], meta.block_table.data_ptr(), meta.max_blocks,
+             0 if token_list is None else token_list.data_ptr(), n, meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(),
+             meta.q_len.data_ptr(), meta.ctx_len.data_ptr(), nh, nkv, dk, dv, page_size, k.shape[0], int(window),
+             int(keep_first), float(softcap or 0.0), float(scale))
+
+    if meta.num_single == t and not meta.num_multi:
+        return singles(None, t)                                 # a decoding step
     # portions of prompts in bfloat16, at the sizes it has: tiles of queries on the matrix cores
-    if (meta.tiles is not None and meta.num_tiles and meta.tile_rows == MASKED_TILE_ROWS and k.dtype is torch.bfloat16
-            and out.dtype is torch.bfloat16 and masked_tiles_take(dk, dv) and k.shape[3] % 8 == 0 and v.shape[3] % 8 == 0
-            and q_token_stride % 4 == 0 and q_head_stride % 4 == 0 and q.data_ptr() % 16 == 0):
+    if (fast and meta.tiles is not None and meta.num_tiles and meta.tile_rows == MASKED_TILE_ROWS and masked_tiles_take(dk, dv)
+            and meta.num_single + meta.num_multi == t):
         _run("attention_masked", "li_masked_attention_tiles", q.data_ptr(), int(q_token_stride), int(q_head_stride),
              out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3], meta.block_table.data_ptr(), meta.max_blocks,
              meta.tiles.data_ptr(), meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale))
         if meta.num_single:
-            general(meta.single_tokens, meta.num_single)       # (a list is there: the batch has tokens of both kinds)
+            singles(meta.single_tokens, meta.num_single)       # (a list is there: the batch has tokens of both kinds)
         return
     general(None, t)
 
 
 MASKED_TILE_ROWS = 32         # queries of one request that a block of the matrix-core kernel takes
+
+
+def masked_single_takes(dk: int, dv: int) -> bool:
+    """Whether the kernel for single tokens has these key and value sizes (bfloat16)."""
+    f = _fn_cache.get(("attention_masked", "li_masked_attention_single_takes"))
+    if f is None:
+        f = build.load("attention_masked").li_masked_attention_single_takes
+        f.argtypes, f.restype = [c_int, c_int], c_int
+        _fn_cache[("attention_masked", "li_masked_attention_single_takes")] = f
+    return bool(f(int(dk), int(dv)))
 
 
 def masked_tiles_take(dk: int, dv: int) -> bool:

@@ -294,6 +294,12 @@ def _close(got, ref, dtype):
     ([(200, 130), (40, 40)], 7, 1, 96, 64, 16, 0, 0, 10.0),            # seven heads on one kv head, no window
     ([(300, 200)], 4, 2, 64, 128, 32, 100, 33, 0.0),
     ([(150, 150), (500, 35)], 3, 1, 320, 256, 16, 64, 1, 0.0),
+    # decoding steps at sizes that the kernel for single tokens takes in bfloat16 (1, 2 and 4 heads a block)
+    ([(700, 1), (90, 1), (3, 1), (41, 1), (1, 1)], 12, 2, 128, 128, 16, 200, 4, 30.0),
+    ([(700, 1), (33, 1)], 7, 1, 64, 64, 8, 0, 0, 0.0),
+    ([(300, 1), (130, 1), (64, 1)], 3, 3, 96, 64, 16, 40, 2, 0.0),
+    ([(1500, 1), (100, 1)], 5, 1, 320, 256, 16, 1024, 0, 0.0),
+    ([(260, 1), (17, 1)], 8, 2, 192, 128, 32, 100, 40, 5.0),
 ])
 def test_masked_attention_against_the_plain_attention(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap):
     got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3)
@@ -305,6 +311,8 @@ def test_values_that_are_the_first_columns_of_the_keys_rows(dtype):
     got, ref = _masked_case(dtype, [(120, 50), (77, 1)], 6, 1, 56, 40, 16, 30, 0, 0.0, seed=4, shared_rows=True)
     _close(got, ref, dtype)
     got, ref = _masked_case(dtype, [(400, 70), (77, 1), (33, 33)], 6, 1, 160, 128, 16, 90, 0, 0.0, seed=5, shared_rows=True)
+    _close(got, ref, dtype)
+    got, ref = _masked_case(dtype, [(400, 1), (77, 1), (1, 1)], 4, 1, 160, 128, 16, 90, 0, 0.0, seed=6, shared_rows=True)
     _close(got, ref, dtype)
 
 
