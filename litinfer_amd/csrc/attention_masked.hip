@@ -213,6 +213,14 @@ extern "C" int li_masked_attention(const float* q, int q_token_stride, int q_hea
 // {16 s + 4 h + i, 16 s + 8 + 4 h + i : i < 4} side by side: the values are written to LDS transposed and in that
 // order.  The visible keys of a tile are its kept first positions and the window of its first to its last query;
 // they are walked as one list (`visible_key`), 32 at a time.
+// exponential and tanh by the hardware's exp2 and reciprocal (relative error about 2^-22: the bfloat16 kernels
+// round their probabilities to 8 bits anyway; the float32 path keeps expf and tanhf)
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float fast_tanh(float x) {
+    const float e = __builtin_amdgcn_exp2f(fminf(x, 40.f) * 2.8853900817779268f);        // exp(2x)
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
 typedef __bf16 ma_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float ma_f32x16 __attribute__((ext_vector_type(16)));
 union ma_frag8 { uint4 raw; uint32_t w[4]; ma_bf16x8 v; };
@@ -246,6 +254,7 @@ __global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
     const int head = kvh * rep + (active ? hh : 0);
     const int pq = p0 + ql;                                               // this lane's query (ql >= ntok: none)
     const int lq = (window > 0) ? pq - window + 1 : 0;
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
 
     ma_frag8 qf[KS];
     {
@@ -316,7 +325,7 @@ __global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
             const int i = i0 + 8 * (r >> 2) + 4 * h + (r & 3);
             const int key = visible_key(i, n_first, lo_min);
             float sc = sv[r] * scale;
-            if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
+            if (softcap > 0.f) sc = softcap * fast_tanh(sc * inv_cap);
             const bool see = i < n_keys && rows[8 * (r >> 2) + 4 * h + (r & 3)] >= 0 && key <= pq && (key >= lq || key < keep_first);
             sv[r] = see ? sc : -INFINITY;
             mx = fmaxf(mx, sv[r]);
@@ -324,10 +333,10 @@ __global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
         mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
         const float mn = fmaxf(m, mx);
         const float ms = (mn == -INFINITY) ? 0.f : mn;                    // a query may see no key of this block
-        const float alpha = (m == -INFINITY) ? 1.f : expf(m - ms);        // (m = -inf: nothing summed yet)
+        const float alpha = (m == -INFINITY) ? 1.f : fast_exp(m - ms);        // (m = -inf: nothing summed yet)
         float psum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { sv[r] = expf(sv[r] - ms); psum += sv[r]; }
+        for (int r = 0; r < 16; ++r) { sv[r] = fast_exp(sv[r] - ms); psum += sv[r]; }
         l = l * alpha + psum;
         m = mn;
 #pragma unroll
@@ -418,18 +427,31 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_list,
     const int* __restrict__ seg_of_token, const int* __restrict__ q_start, const int* __restrict__ q_len,
     const int* __restrict__ ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages, int window,
-    int keep_first, float softcap, float scale) {
-    extern __shared__ float join[];                 // [4 waves][RH][dv + 2]
+    int keep_first, float softcap, float scale, int tab_cap, int pshift, int nsplit, float* __restrict__ parts) {
+    extern __shared__ float join[];                 // [4 waves][RH][dv + 2], then tab_cap table entries
+    int* tab = (int*)(join + (size_t)4 * RH * (dv + 2));
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, g = lane >> 3, j = lane & 7;
     const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, kvh = blockIdx.y;
-    const int rep = nh / nkv, hfirst = blockIdx.z * RH;
+    const int rep = nh / nkv, hfirst = (blockIdx.z / nsplit) * RH, sp = blockIdx.z % nsplit;
     const int nheads = rep - hfirst < RH ? rep - hfirst : RH;
     const int s = seg_of_token[t];
     const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int n_first = keep_first < lo ? keep_first : lo;
-    const int n_keys = n_first + (p - lo + 1);
+    const int n_all = n_first + (p - lo + 1);
+    // this block's share of the visible keys (split sp of nsplit)
+    const int i_begin = (int)((long)n_all * sp / nsplit), n_keys = (int)((long)n_all * (sp + 1) / nsplit);
     const int* table = block_table + (size_t)s * max_blocks;
+    // the pages of the visible keys in LDS (the window's blocks, then the kept first blocks), so that a key's row
+    // costs no trip to memory before its own; a table too long for the room given is read where it lies
+    const int b_lo = pshift >= 0 ? lo >> pshift : lo / page_size, b_hi = pshift >= 0 ? p >> pshift : p / page_size;
+    const int nb_w = b_hi - b_lo + 1, nb_k = n_first > 0 ? (n_first - 1) / page_size + 1 : 0;
+    const bool in_lds = nb_w + nb_k <= tab_cap;
+    if (in_lds) {
+        for (int i = threadIdx.x; i < nb_w; i += 256) tab[i] = table[b_lo + i];
+        for (int i = threadIdx.x; i < nb_k; i += 256) tab[nb_w + i] = table[i];
+    }
+    __syncthreads();
 
     float qr[RH][NPK][8];
 #pragma unroll
@@ -455,32 +477,43 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc[hh][c][e] = 0.f;
     }
-    for (int i0 = 0; i0 < n_keys; i0 += 32 * U) {
-        size_t ro[U];
-        bool ok[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int i = i0 + 32 * u + 8 * w + g;
-            ok[u] = i < n_keys;
-            const int key = visible_key(ok[u] ? i : 0, n_first, lo);
-            const int page = table[key / page_size];
-            ok[u] = ok[u] && page >= 0 && page < num_pages;
-            ro[u] = ok[u] ? (size_t)(page * nkv + kvh) * page_size + key % page_size : 0;      // (row 0 exists: read, not used)
-        }
-        uint4 kp[U][NPK], vp[U][NPV];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int c = 0; c < NPK; ++c) {
-                const int d0 = 8 * (j + 8 * c);
-                kp[u][c] = *reinterpret_cast<const uint4*>(kc + ro[u] * k_row + (d0 < dk ? d0 : 0));
-            }
-#pragma unroll
-            for (int c = 0; c < NPV; ++c) {
-                const int d0 = 8 * (j + 8 * c);
-                vp[u][c] = *reinterpret_cast<const uint4*>(vc + ro[u] * v_row + (d0 < dv ? d0 : 0));
-            }
-        }
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+    // the rows of a round's keys (a key past the last: row 0, read and not used) and their pieces; the next round's
+    // are asked for before this round's are used, without a condition (a load under a condition would make every
+    // later use wait for all loads)
+    size_t ro[U];
+    bool ok[U];
+    uint4 kp[U][NPK], vp[U][NPV];
+#define MS_ROWS(I0, RO, OK)                                                                                          \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                                  \
+        const int i = (I0) + 32 * u + 8 * w + g;                                                                     \
+        OK[u] = i < n_keys;                                                                                          \
+        const int ii = OK[u] ? i : 0;                                                                                \
+        const int key = visible_key(ii, n_first, lo);                                                                \
+        const int blk = pshift >= 0 ? key >> pshift : key / page_size;                                               \
+        const int page = in_lds ? tab[ii < n_first ? nb_w + blk : blk - b_lo] : table[blk];                          \
+        OK[u] = OK[u] && page >= 0 && page < num_pages;                                                              \
+        RO[u] = OK[u] ? (size_t)(page * nkv + kvh) * page_size + (key - blk * page_size) : 0;                        \
+    }
+#define MS_FETCH(RO, KP, VP)                                                                                         \
+    _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                                  \
+        _Pragma("unroll") for (int c = 0; c < NPK; ++c) {                                                            \
+            const int d0 = 8 * (j + 8 * c);                                                                          \
+            KP[u][c] = *reinterpret_cast<const uint4*>(kc + RO[u] * k_row + (d0 < dk ? d0 : 0));                     \
+        }                                                                                                            \
+        _Pragma("unroll") for (int c = 0; c < NPV; ++c) {                                                            \
+            const int d0 = 8 * (j + 8 * c);                                                                          \
+            VP[u][c] = *reinterpret_cast<const uint4*>(vc + RO[u] * v_row + (d0 < dv ? d0 : 0));                     \
+        }                                                                                                            \
+    }
+    MS_ROWS(i_begin, ro, ok)
+    MS_FETCH(ro, kp, vp)
+    for (int i0 = i_begin; i0 < n_keys; i0 += 32 * U) {
+        size_t ro2[U];
+        bool ok2[U];
+        uint4 kp2[U][NPK], vp2[U][NPV];
+        MS_ROWS(i0 + 32 * U, ro2, ok2)
+        MS_FETCH(ro2, kp2, vp2)
         float sc[U][RH];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -498,7 +531,7 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
                 d += __shfl_xor(d, 2, LI_WAVE);
                 d += __shfl_xor(d, 4, LI_WAVE);
                 d *= scale;
-                if (softcap > 0.f) d = softcap * tanhf(d / softcap);
+                if (softcap > 0.f) d = softcap * fast_tanh(d * inv_cap);
                 sc[u][hh] = ok[u] ? d : -INFINITY;
             }
         }
@@ -509,10 +542,10 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
             for (int u = 1; u < U; ++u) mx = fmaxf(mx, sc[u][hh]);
             const float mn = fmaxf(m[hh], mx);
             const float ms = (mn == -INFINITY) ? 0.f : mn;
-            const float alpha = (m[hh] == -INFINITY) ? 0.f : expf(m[hh] - ms);
+            const float alpha = (m[hh] == -INFINITY) ? 0.f : fast_exp(m[hh] - ms);
             float pu[U], psum = 0.f;
 #pragma unroll
-            for (int u = 0; u < U; ++u) { pu[u] = expf(sc[u][hh] - ms); psum += pu[u]; }
+            for (int u = 0; u < U; ++u) { pu[u] = fast_exp(sc[u][hh] - ms); psum += pu[u]; }
             l[hh] = l[hh] * alpha + psum;
             m[hh] = mn;
 #pragma unroll
@@ -531,7 +564,17 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
                 for (int e = 0; e < 8; ++e) acc[hh][c][e] = a8[e];
             }
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            ok[u] = ok2[u];
+#pragma unroll
+            for (int c = 0; c < NPK; ++c) kp[u][c] = kp2[u][c];
+#pragma unroll
+            for (int c = 0; c < NPV; ++c) vp[u][c] = vp2[u][c];
+        }
     }
+#undef MS_ROWS
+#undef MS_FETCH
     // the groups of a wave
 #pragma unroll
     for (int off = 8; off < 64; off <<= 1) {
@@ -577,7 +620,33 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
             a += r[d] * f;
             ll += r[dv + 1] * f;
         }
-        out[((size_t)t * nh + kvh * rep + hfirst + hh) * dv + d].bits = float_to_bf16(ll != 0.f ? a / ll : 0.f);
+        const int head = kvh * rep + hfirst + hh;
+        if (nsplit == 1) {
+            out[((size_t)t * nh + head) * dv + d].bits = float_to_bf16(ll != 0.f ? a / ll : 0.f);
+        } else {                                    // this split's sums, maximum and sum of weights: joined by the kernel behind
+            float* part = parts + (((size_t)blockIdx.x * nh + head) * nsplit + sp) * (dv + 2);
+            part[d] = a;
+            if (d == 0) { part[dv] = mm; part[dv + 1] = ll; }
+        }
+    }
+}
+
+// joins the splits of every (token, head) in split order: a block a (token, head)
+__global__ void masked_attention_join_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
+                                             const int* __restrict__ token_list, int nh, int dv, int nsplit) {
+    const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, head = blockIdx.y;
+    const float* base = parts + ((size_t)blockIdx.x * nh + head) * nsplit * (dv + 2);
+    float mm = -INFINITY;
+    for (int x = 0; x < nsplit; ++x) mm = fmaxf(mm, base[(size_t)x * (dv + 2) + dv]);
+    for (int d = threadIdx.x; d < dv; d += blockDim.x) {
+        float a = 0.f, ll = 0.f;
+        for (int x = 0; x < nsplit; ++x) {
+            const float* r = base + (size_t)x * (dv + 2);
+            const float f = (r[dv] == -INFINITY) ? 0.f : expf(r[dv] - mm);
+            a += r[d] * f;
+            ll += r[dv + 1] * f;
+        }
+        out[((size_t)t * nh + head) * dv + d].bits = float_to_bf16(ll != 0.f ? a / ll : 0.f);
     }
 }
 
@@ -588,38 +657,58 @@ extern "C" int li_masked_attention_single_takes(int dk, int dv) {
     return (npk <= 2 && npv <= 2) || (npk == 3 && npv == 2) || (npk == 4 && npv == 4) || (npk == 5 && npv == 4) || (npk == 4 && npv == 3);
 }
 
+// blocks that a call launches per split (the host sizes the number of splits by it)
+extern "C" int li_masked_attention_single_blocks(int n_tokens, int nh, int nkv, int dk, int dv) {
+    const int rep = nh / nkv, npk = (dk + 63) / 64, npv = (dv + 63) / 64;
+    const int rh = (npk + npv > 6) ? (rep >= 2 ? 2 : 1) : (rep >= 4 && (rep % 4 == 0 || rep % 4 == 3 || rep > 8)) ? 4 : rep >= 2 ? 2 : 1;
+    return n_tokens * nkv * ((rep + rh - 1) / rh);
+}
+
 extern "C" int li_masked_attention_single(const float* q, int q_token_stride, int q_head_stride, void* out, const void* kc,
                                           const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
                                           const int* token_list, int n_tokens, const int* seg_of_token, const int* q_start,
                                           const int* q_len, const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size,
                                           int num_pages, int window, int keep_first, float softcap, float scale,
-                                          hipStream_t stream) {
+                                          int nsplit, float* parts, long parts_floats, hipStream_t stream) {
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
         window < 0 || keep_first < 0 || max_blocks <= 0 || num_pages <= 0 || k_row % 8 || v_row % 8 || q_token_stride % 4 ||
         q_head_stride % 4 || ((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) % 16 || !li_masked_attention_single_takes(dk, dv))
         return LI_ERR_SIZE;
     const int rep = nh / nkv, npk = (dk + 63) / 64, npv = (dv + 63) / 64;
     const int rh = (npk + npv > 6) ? (rep >= 2 ? 2 : 1) : (rep >= 4 && (rep % 4 == 0 || rep % 4 == 3 || rep > 8)) ? 4 : rep >= 2 ? 2 : 1;
-    const dim3 grid(n_tokens, nkv, (rep + rh - 1) / rh);
-    const size_t lds = (size_t)4 * rh * (dv + 2) * 4;
+    if (nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!parts || parts_floats < (long)n_tokens * nh * nsplit * (dv + 2)))) return LI_ERR_SIZE;
+    const dim3 grid(n_tokens, nkv, ((rep + rh - 1) / rh) * nsplit);
+    // room for the pages of one query's visible keys: the window's and the kept ones, or the whole table's width
+    long cap = window > 0 ? (long)window / page_size + 3 + (keep_first + page_size - 1) / page_size : (long)max_blocks;
+    if (cap > 12288) cap = 0;                       // (longer tables are read where they lie)
+    const int tab_cap = (int)cap;
+    int pshift = -1;
+    for (int b = 0; b < 31; ++b) if (page_size == (1 << b)) pshift = b;
+    const size_t lds = (size_t)4 * rh * (dv + 2) * 4 + (size_t)tab_cap * 4;
 #define MS_GO(K, V, R, UU)                                                                                                  \
     masked_attention_single_kernel<K, V, R, UU><<<grid, 256, lds, stream>>>(                                                \
         q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table,    \
         max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, nh, nkv, dk, dv, page_size, num_pages, window,       \
-        keep_first, softcap, scale)
+        keep_first, softcap, scale, tab_cap, pshift, nsplit, parts)
+#define MS_JOIN                                                                                                             \
+    if (nsplit > 1)                                                                                                         \
+        masked_attention_join_kernel<<<dim3(n_tokens, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, token_list, nh, dv, nsplit);
 #define MS_SMALL(K, V)                                                                                                      \
     if (npk == K && npv == V) {                                                                                             \
         if (rh == 4) MS_GO(K, V, 4, 4); else if (rh == 2) MS_GO(K, V, 2, 4); else MS_GO(K, V, 1, 4);                        \
+        MS_JOIN                                                                                                             \
         return li_launch_status();                                                                                          \
     }
 #define MS_LARGE(K, V)                                                                                                      \
     if (npk == K && npv == V) {                                                                                             \
         if (rh == 2) MS_GO(K, V, 2, 2); else MS_GO(K, V, 1, 2);                                                             \
+        MS_JOIN                                                                                                             \
         return li_launch_status();                                                                                          \
     }
     MS_SMALL(1, 1) MS_SMALL(2, 1) MS_SMALL(1, 2) MS_SMALL(2, 2) MS_SMALL(3, 2)
     MS_LARGE(4, 4) MS_LARGE(5, 4) MS_LARGE(4, 3)
 #undef MS_GO
+#undef MS_JOIN
 #undef MS_SMALL
 #undef MS_LARGE
     return LI_ERR_SIZE;
@@ -644,16 +733,19 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
         xs[i] = tt < nt ? load_as_float(x + (size_t)(t0 + tt) * x_token_stride + (size_t)h * x_head_stride + k) : 0.f;
     }
     __syncthreads();
-    for (int j = blockIdx.z * 256 + threadIdx.x; j < n_out; j += gridDim.z * 256) {
-        const TM* row = m + ((size_t)h * n_out + j) * n_in;
+    // four neighbouring threads share an output: each takes every fourth piece of the matrix row
+    constexpr int E = VEC ? 16 / (int)sizeof(TM) : 1;
+    const int part = threadIdx.x & 3;
+    for (int j = blockIdx.z * 64 + (threadIdx.x >> 2); j < n_out + 63; j += gridDim.z * 64) {       // (whole groups of four go round together)
+        const bool on = j < n_out;
+        const TM* row = m + ((size_t)h * n_out + (on ? j : 0)) * n_in;
         float acc[HL_TOK];
 #pragma unroll
         for (int tt = 0; tt < HL_TOK; ++tt) acc[tt] = 0.f;
-        if constexpr (VEC) {
-            constexpr int E = 16 / sizeof(TM);
-            for (int k = 0; k < n_in; k += E) {
+        for (int k = part * E; k < n_in; k += 4 * E) {
+            float wv[E];
+            if constexpr (VEC) {
                 const uint4 raw = *reinterpret_cast<const uint4*>(row + k);
-                float wv[E];
                 if constexpr (sizeof(TM) == 2) {
                     const uint32_t r4[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -665,20 +757,22 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
                     wv[0] = __uint_as_float(raw.x); wv[1] = __uint_as_float(raw.y);
                     wv[2] = __uint_as_float(raw.z); wv[3] = __uint_as_float(raw.w);
                 }
-#pragma unroll
-                for (int e = 0; e < E; ++e)
-#pragma unroll
-                    for (int tt = 0; tt < HL_TOK; ++tt) acc[tt] = fmaf(wv[e], xs[tt * n_in + k + e], acc[tt]);
+            } else {
+                wv[0] = load_as_float(row + k);
             }
-        } else {
-            for (int k = 0; k < n_in; ++k) {
-                const float wv = load_as_float(row + k);
 #pragma unroll
-                for (int tt = 0; tt < HL_TOK; ++tt) acc[tt] = fmaf(wv, xs[tt * n_in + k], acc[tt]);
-            }
+            for (int e = 0; e < E; ++e)
+#pragma unroll
+                for (int tt = 0; tt < HL_TOK; ++tt) acc[tt] = fmaf(wv[e], xs[tt * n_in + k + e], acc[tt]);
         }
-        for (int tt = 0; tt < nt; ++tt)
-            store_from_float(out + (size_t)(t0 + tt) * o_token_stride + (size_t)h * o_head_stride + j, acc[tt]);
+#pragma unroll
+        for (int tt = 0; tt < HL_TOK; ++tt) {
+            acc[tt] += __shfl_xor(acc[tt], 1, LI_WAVE);
+            acc[tt] += __shfl_xor(acc[tt], 2, LI_WAVE);
+        }
+        if (on && part == 0)
+            for (int tt = 0; tt < nt; ++tt)
+                store_from_float(out + (size_t)(t0 + tt) * o_token_stride + (size_t)h * o_head_stride + j, acc[tt]);
     }
 }
 
@@ -754,7 +848,7 @@ extern "C" int li_headwise_linear(const void* x, int x_dtype, long x_token_strid
         else if (x_dtype == LI_BF16 && out_dtype == LI_F32) took = headwise_mfma<bf16_t, float>(x, x_token_stride, x_head_stride, m, out, o_token_stride, o_head_stride, T_, nh, n_out, n_in, stream);
         if (took) return li_launch_status();
     }
-    const int zs = (n_out + 255) / 256;
+    const int zs = (n_out + 63) / 64;
     const dim3 grid((T_ + HL_TOK - 1) / HL_TOK, nh, zs < 64 ? zs : 64);
     const size_t lds = (size_t)HL_TOK * n_in * 4;
 #define HL_GO(TX, TM, TO)                                                                                                  \

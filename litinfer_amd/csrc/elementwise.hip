@@ -641,13 +641,19 @@ extern "C" int li_qk_norm_pairs_store(float* qkv, int row_stride, int nh, int nk
     if (T <= 0 || nh <= 0 || nkv <= 0 || dk <= 0 || dv <= 0 || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > dk ||
         row_stride < nh * dk + nkv * (dk + dv) || page_size <= 0)
         return LI_ERR_SIZE;
-    if (cache_dtype == LI_F32)
-        qk_norm_pairs_store_kernel<float, 256><<<T, 256, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps,
-                                                                      cosv, sinv, slot_map, (float*)kc, (float*)vc, page_size, store);
-    else if (cache_dtype == LI_BF16)
-        qk_norm_pairs_store_kernel<bf16_t, 256><<<T, 256, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps,
-                                                                       cosv, sinv, slot_map, (bf16_t*)kc, (bf16_t*)vc, page_size, store);
+    // few rows (a decoding step): 1024 threads a row, so that the one row is gone through with the least latency
+    const bool wide = T < 256 && nh * dk > 1024;
+#define LI_QK(TC)                                                                                                            \
+    {                                                                                                                        \
+        if (wide) qk_norm_pairs_store_kernel<TC, 1024><<<T, 1024, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps, \
+                                                                              cosv, sinv, slot_map, (TC*)kc, (TC*)vc, page_size, store); \
+        else qk_norm_pairs_store_kernel<TC, 256><<<T, 256, 0, stream>>>(qkv, row_stride, nh, nkv, dk, dv, rotary_dim, wq, wk, eps,  \
+                                                                        cosv, sinv, slot_map, (TC*)kc, (TC*)vc, page_size, store);  \
+    }
+    if (cache_dtype == LI_F32) LI_QK(float)
+    else if (cache_dtype == LI_BF16) LI_QK(bf16_t)
     else return LI_ERR_DTYPE;
+#undef LI_QK
     return li_launch_status();
 }
 

@@ -47,7 +47,7 @@ _SIGNATURES = {
     },
     "attention_masked": {
         "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I],
-        "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F],
+        "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
         "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F],
         "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I],
     },
@@ -482,9 +482,21 @@ def latent_norm_pairs_store(qd: torch.Tensor, nh: int, dn: int, dr: int, rank: i
              int(cache is not None), t)
 
 
+MASKED_SINGLE_BLOCKS = 512    # blocks of four waves that the kernel for single tokens is cut into at least, where the keys allow
+
+
+def _single_blocks(n: int, nh: int, nkv: int, dk: int, dv: int) -> int:
+    f = _fn_cache.get(("attention_masked", "li_masked_attention_single_blocks"))
+    if f is None:
+        f = build.load("attention_masked").li_masked_attention_single_blocks
+        f.argtypes, f.restype = [c_int] * 5, c_int
+        _fn_cache[("attention_masked", "li_masked_attention_single_blocks")] = f
+    return max(1, int(f(n, nh, nkv, dk, dv)))
+
+
 def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, out: torch.Tensor, k: torch.Tensor,
                      v: torch.Tensor, meta, nh: int, nkv: int, dk: int, dv: int, page_size: int, window: int,
-                     keep_first: int, softcap: float, scale: float) -> None:
+                     keep_first: int, softcap: float, scale: float, ws=None) -> None:
     """Attention of every token of the step over its request's cached keys: position p sees j <= p with
     p - j < window (0: all) or j < keep_first; scores (q . k) * scale, then softcap * tanh(score / softcap)
     where softcap > 0; softmax and sums in float32.  q: a float32 tensor in which head h of token t starts at
@@ -521,11 +533,19 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
         # single tokens in bfloat16, at the sizes it has: rows spread over lanes, a row read once for a group's heads
         if not (fast and masked_single_takes(dk, dv)):
             return general(token_list, n)
+        # few blocks against many keys: the keys are cut into splits, each a block of its own, and joined by a second
+        # kernel (the number follows the table's width or the window, not the contexts: a recorded step keeps it)
+        blocks = _single_blocks(n, nh, nkv, dk, dv)
+        nsplit = max(1, min(-(-MASKED_SINGLE_BLOCKS // blocks), bound // 128, 32)) if ws is not None else 1
+        parts, parts_n = 0, 0
+        if nsplit > 1:
+            buf = ws.buffer("masked_attention.parts", (n * nh * nsplit * (dv + 2),), torch.float32)
+            parts, parts_n = buf.data_ptr(), buf.numel()
         _run("attention_masked", "li_masked_attention_single", q.data_ptr(), int(q_token_stride), int(q_head_stride),
              out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3], meta.block_table.data_ptr(), meta.max_blocks,
              0 if token_list is None else token_list.data_ptr(), n, meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(),
              meta.q_len.data_ptr(), meta.ctx_len.data_ptr(), nh, nkv, dk, dv, page_size, k.shape[0], int(window),
-             int(keep_first), float(softcap or 0.0), float(scale))
+             int(keep_first), float(softcap or 0.0), float(scale), nsplit, parts, parts_n)
 
     if meta.num_single == t and not meta.num_multi:
         return singles(None, t)                                 # a decoding step

@@ -101,7 +101,7 @@ class MaskedAttention(Mixer):
         attn = ctx.ws.buffer("attn.out", (t, self.nh * self.dv), self.rt.dtype)
         ops.masked_attention(qkv, qkv.stride(0), self.dk, attn, cache.k, cache.v, ctx.attention_meta(cache.group),
                              self.nh, self.nkv, self.dk, self.dv, cache.page_size, self.window, self.keep_first,
-                             self.softcap, self.scale)
+                             self.softcap, self.scale, ws=ctx.ws)
         residual.add_linear(self.out, attn)
 
 
@@ -177,7 +177,8 @@ class LatentAttention(Mixer):
         ops.headwise_linear(qd, qd.stride(0), dn + dr, self.to_latent, qfull, nh * (rank + dr), rank + dr, t)
         summed = ctx.ws.buffer("latent.summed", (t, nh * rank), self.rt.dtype)
         ops.masked_attention(qfull, nh * (rank + dr), rank + dr, summed, rows, rows, ctx.attention_meta(cache.group),
-                             nh, 1, rank + dr, rank, cache.page_size, self.window, self.keep_first, self.softcap, self.scale)
+                             nh, 1, rank + dr, rank, cache.page_size, self.window, self.keep_first, self.softcap, self.scale,
+                             ws=ctx.ws)
         heads = ctx.ws.buffer("attn.out", (t, nh * self.dv), self.rt.dtype)
         ops.headwise_linear(summed, nh * rank, rank, self.from_latent, heads, nh * self.dv, self.dv, t)
         residual.add_linear(self.out, heads)

@@ -258,7 +258,9 @@ def _masked_case(dtype, seg_specs, nh, nkv, dk, dv, page, window, keep_first, so
     qd = q.to(DEV).contiguous()
     kd = kc.to(DEV)
     vd = kd if shared_rows else vc.to(DEV)
-    ops.masked_attention(qd, nh * dk, dk, out, kd, vd, meta, nh, nkv, dk, dv, page, window, keep_first, softcap, scale)
+    from litinfer_amd.engine.workspace import Workspace
+    ops.masked_attention(qd, nh * dk, dk, out, kd, vd, meta, nh, nkv, dk, dv, page, window, keep_first, softcap, scale,
+                         ws=Workspace(DEV))
     refs, o = [], 0
     rep = nh // nkv
     for s, (c, ql) in enumerate(seg_specs):
@@ -300,6 +302,8 @@ def _close(got, ref, dtype):
     ([(300, 1), (130, 1), (64, 1)], 3, 3, 96, 64, 16, 40, 2, 0.0),
     ([(1500, 1), (100, 1)], 5, 1, 320, 256, 16, 1024, 0, 0.0),
     ([(260, 1), (17, 1)], 8, 2, 192, 128, 32, 100, 40, 5.0),
+    ([(3000, 1), (5, 1), (129, 1)], 4, 2, 128, 128, 16, 0, 0, 0.0),           # many splits of the keys, some of them empty
+    ([(2500, 1), (300, 1)], 6, 1, 160, 128, 16, 2000, 3, 0.0),
 ])
 def test_masked_attention_against_the_plain_attention(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap):
     got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3)
