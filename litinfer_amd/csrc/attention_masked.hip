@@ -238,7 +238,7 @@ __global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
     constexpr int NT = MT_WAVES * 64;
     __shared__ __attribute__((aligned(16))) uint16_t Ks[32 * KROW];       // [key place][dimension]
     __shared__ __attribute__((aligned(16))) uint16_t Vt[DV * MT_VS];      // [value column][key place, permuted]
-    __shared__ int rows[32];                                              // the cache row of each key place, -1: none
+    __shared__ int rows[3][32];                                           // the cache row of each key place of three blocks in turn, -1: none
     const int tile = blockIdx.x, kvh = blockIdx.y;
     const int s = tiles[4 * tile], t0 = tiles[4 * tile + 1], ntok = tiles[4 * tile + 2];
     const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);             // position of the tile's first query
@@ -273,91 +273,139 @@ __global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
     float m = -INFINITY, l = 0.f;
+    const int lq_last = (window > 0) ? p_last - window + 1 : 0;           // the highest lower edge among the tile's queries
 
-    for (int i0 = 0; i0 < n_keys; i0 += 32) {
-        __syncthreads();                                                  // the block before has been read
-        if (threadIdx.x < 32) {
-            const int i = i0 + threadIdx.x;
-            int ro = -1;
-            if (i < n_keys) {
-                const int key = visible_key(i, n_first, lo_min);
-                const int page = table[key / page_size];
-                if (page >= 0 && page < num_pages) ro = (page * nkv + kvh) * page_size + key % page_size;
-            }
-            rows[threadIdx.x] = ro;
-        }
-        __syncthreads();
-        for (int i = threadIdx.x; i < 32 * (DK / 8); i += NT) {
-            const int kk = i / (DK / 8), c = i % (DK / 8), ro = rows[kk];
-            uint4 raw = {0u, 0u, 0u, 0u};
-            if (ro >= 0) raw = *reinterpret_cast<const uint4*>(kc + (size_t)ro * k_row + 8 * c);
-            *reinterpret_cast<uint4*>(&Ks[kk * KROW + 8 * c]) = raw;
-        }
-        for (int i = threadIdx.x; i < 32 * (DV / 8); i += NT) {
-            const int kk = i % 32, c = i / 32, ro = rows[kk];             // (neighbouring threads: neighbouring key places)
-            uint4 raw = {0u, 0u, 0u, 0u};
-            if (ro >= 0) raw = *reinterpret_cast<const uint4*>(vc + (size_t)ro * v_row + 8 * c);
-            const int k16 = kk & 15, rem = k16 & 7;
-            const int place = (kk & 16) + 8 * (rem >> 2) + 4 * (k16 >> 3) + (rem & 3);
-            const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                Vt[(8 * c + 2 * e) * MT_VS + place] = (uint16_t)(wv[e] & 0xffffu);
-                Vt[(8 * c + 2 * e + 1) * MT_VS + place] = (uint16_t)(wv[e] >> 16);
-            }
-        }
-        __syncthreads();
-        if (!active) continue;
-        // ---- S^T = K Q^T
-        ma_f32x16 sv;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sv[r] = 0.f;
-#pragma unroll
-        for (int st = 0; st < KS; ++st) {
-            ma_frag8 kf;
-            kf.raw = *reinterpret_cast<const uint4*>(&Ks[ql * KROW + 16 * st + 8 * h]);
-            sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[st].v, sv, 0, 0, 0);
-        }
-        // ---- scale, cap, mask, softmax over the keys of this lane's query
-        float mx = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int i = i0 + 8 * (r >> 2) + 4 * h + (r & 3);
-            const int key = visible_key(i, n_first, lo_min);
-            float sc = sv[r] * scale;
-            if (softcap > 0.f) sc = softcap * fast_tanh(sc * inv_cap);
-            const bool see = i < n_keys && rows[8 * (r >> 2) + 4 * h + (r & 3)] >= 0 && key <= pq && (key >= lq || key < keep_first);
-            sv[r] = see ? sc : -INFINITY;
-            mx = fmaxf(mx, sv[r]);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
-        const float mn = fmaxf(m, mx);
-        const float ms = (mn == -INFINITY) ? 0.f : mn;                    // a query may see no key of this block
-        const float alpha = (m == -INFINITY) ? 1.f : fast_exp(m - ms);        // (m = -inf: nothing summed yet)
-        float psum = 0.f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { sv[r] = fast_exp(sv[r] - ms); psum += sv[r]; }
-        l = l * alpha + psum;
-        m = mn;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
-        ma_frag8 pf[2];
-#pragma unroll
-        for (int st = 0; st < 2; ++st)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pf[st].w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int st = 0; st < 2; ++st) {
-                ma_frag8 vf;
-                vf.raw = *reinterpret_cast<const uint4*>(&Vt[(32 * dt + ql) * MT_VS + 16 * st + 8 * h]);
-                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
-            }
+    // The cache row of key place tid of the block of keys that starts at list index i0 (threads 0..31).
+    auto row_of = [&](int i0) -> int {
+        const int i = i0 + (int)threadIdx.x;
+        if (i >= n_keys) return -1;
+        const int key = visible_key(i, n_first, lo_min);
+        const int page = table[key / page_size];
+        return (page >= 0 && page < num_pages) ? (page * nkv + kvh) * page_size + key % page_size : -1;
+    };
+    constexpr int NKC = (32 * (DK / 8) + NT - 1) / NT, NVC = (32 * (DV / 8) + NT - 1) / NT;
+    uint4 kreg[NKC], vreg[NVC];
+    // a block's keys and values on their way: from memory into registers (a place without a row reads row 0 and
+    // is zeroed when it is stored) ...
+#define MT_LOAD(RB)                                                                                                   \
+    _Pragma("unroll") for (int n = 0; n < NKC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        const int kk = (i / (DK / 8)) & 31, c = i % (DK / 8), ro = rows[RB][kk];                                      \
+        kreg[n] = *reinterpret_cast<const uint4*>(kc + (size_t)(ro >= 0 ? ro : 0) * k_row + 8 * c);                   \
+    }                                                                                                                 \
+    _Pragma("unroll") for (int n = 0; n < NVC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        const int kk = i % 32, c = (i / 32) % (DV / 8), ro = rows[RB][kk];                                            \
+        vreg[n] = *reinterpret_cast<const uint4*>(vc + (size_t)(ro >= 0 ? ro : 0) * v_row + 8 * c);                   \
     }
+    // ... and from the registers into LDS: keys as they are, values transposed and in the operand's key order
+#define MT_STORE(RB)                                                                                                  \
+    _Pragma("unroll") for (int n = 0; n < NKC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        if (i < 32 * (DK / 8)) {                                                                                      \
+            const int kk = i / (DK / 8), c = i % (DK / 8);                                                            \
+            *reinterpret_cast<uint4*>(&Ks[kk * KROW + 8 * c]) = rows[RB][kk] >= 0 ? kreg[n] : uint4{0u, 0u, 0u, 0u};  \
+        }                                                                                                             \
+    }                                                                                                                 \
+    _Pragma("unroll") for (int n = 0; n < NVC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        if (i < 32 * (DV / 8)) {                                                                                      \
+            const int kk = i % 32, c = i / 32;                                                                        \
+            const uint4 raw = rows[RB][kk] >= 0 ? vreg[n] : uint4{0u, 0u, 0u, 0u};                                    \
+            const int k16 = kk & 15, rem = k16 & 7;                                                                   \
+            const int place = (kk & 16) + 8 * (rem >> 2) + 4 * (k16 >> 3) + (rem & 3);                                \
+            const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};                                                      \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                           \
+                Vt[(8 * c + 2 * e) * MT_VS + place] = (uint16_t)(wv[e] & 0xffffu);                                    \
+                Vt[(8 * c + 2 * e + 1) * MT_VS + place] = (uint16_t)(wv[e] >> 16);                                    \
+            }                                                                                                         \
+        }                                                                                                             \
+    }
+    const int nblk = (n_keys + 31) / 32;
+    if (threadIdx.x < 32) {
+        rows[0][threadIdx.x] = row_of(0);
+        rows[1][threadIdx.x] = row_of(32);
+    }
+    __syncthreads();
+    MT_LOAD(0)
+    MT_STORE(0)
+    __syncthreads();
+    // block b is in LDS; block b + 1 is asked for before b is worked on, and the rows of b + 2 before that
+    for (int b = 0; b < nblk; ++b) {
+        const int i0 = 32 * b, rb = b % 3, rb1 = (b + 1) % 3, rb2 = (b + 2) % 3;
+        int ro2 = -1;
+        if (threadIdx.x < 32) ro2 = row_of(i0 + 64);
+        MT_LOAD(rb1)                                                      // (past the last block: its rows are -1, row 0 is read and never stored)
+        if (active) {
+            // ---- S^T = K Q^T
+            ma_f32x16 sv;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sv[r] = 0.f;
+#pragma unroll
+            for (int st = 0; st < KS; ++st) {
+                ma_frag8 kf;
+                kf.raw = *reinterpret_cast<const uint4*>(&Ks[ql * KROW + 16 * st + 8 * h]);
+                sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[st].v, sv, 0, 0, 0);
+            }
+            // ---- scale, cap, mask.  A block that every query of the tile sees whole (most are) needs no masks: its
+            // places all have rows, it lies wholly among the kept positions or wholly inside every query's window.
+            const bool whole = i0 + 31 < n_keys && !(i0 < n_first && i0 + 31 >= n_first) && __all(rows[rb][ql] >= 0) &&
+                               (i0 + 31 < n_first || (visible_key(i0 + 31, n_first, lo_min) <= p0 && visible_key(i0, n_first, lo_min) >= lq_last));
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float sc = sv[r] * scale;
+                if (softcap > 0.f) sc = softcap * fast_tanh(sc * inv_cap);
+                sv[r] = sc;
+            }
+            if (!whole) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int place = 8 * (r >> 2) + 4 * h + (r & 3), i = i0 + place;
+                    const int key = visible_key(i, n_first, lo_min);
+                    const bool see = i < n_keys && rows[rb][place] >= 0 && key <= pq && (key >= lq || key < keep_first);
+                    sv[r] = see ? sv[r] : -INFINITY;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sv[r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
+            const float mn = fmaxf(m, mx);
+            const float ms = (mn == -INFINITY) ? 0.f : mn;                    // a query may see no key of this block
+            const float alpha = (m == -INFINITY) ? 1.f : fast_exp(m - ms);    // (m = -inf: nothing summed yet)
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sv[r] = fast_exp(sv[r] - ms); psum += sv[r]; }
+            l = l * alpha + psum;
+            m = mn;
+            if (__any(alpha != 1.f)) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
+            }
+            ma_frag8 pf[2];
+#pragma unroll
+            for (int st = 0; st < 2; ++st)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) pf[st].w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int st = 0; st < 2; ++st) {
+                    ma_frag8 vf;
+                    vf.raw = *reinterpret_cast<const uint4*>(&Vt[(32 * dt + ql) * MT_VS + 16 * st + 8 * h]);
+                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
+                }
+        }
+        __syncthreads();                                                  // block b has been read
+        if (b + 1 < nblk) { MT_STORE(rb1) }
+        if (threadIdx.x < 32) rows[rb2][threadIdx.x] = ro2;
+        __syncthreads();
+    }
+#undef MT_LOAD
+#undef MT_STORE
     if (!active) return;
     l += __shfl_xor(l, 32, LI_WAVE);
     if (ql >= ntok) return;

@@ -482,7 +482,15 @@ def latent_norm_pairs_store(qd: torch.Tensor, nh: int, dn: int, dr: int, rank: i
              int(cache is not None), t)
 
 
-MASKED_SINGLE_BLOCKS = 512    # blocks of four waves that the kernel for single tokens is cut into at least, where the keys allow
+_CUS: Dict[int, int] = {}
+
+
+def _compute_units(device: torch.device) -> int:
+    idx = device.index or 0
+    if idx not in _CUS:
+        _CUS[idx] = int(torch.cuda.get_device_properties(device).multi_processor_count)
+    return _CUS[idx]
+
 
 
 def _single_blocks(n: int, nh: int, nkv: int, dk: int, dv: int) -> int:
@@ -536,7 +544,9 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
         # few blocks against many keys: the keys are cut into splits, each a block of its own, and joined by a second
         # kernel (the number follows the table's width or the window, not the contexts: a recorded step keeps it)
         blocks = _single_blocks(n, nh, nkv, dk, dv)
-        nsplit = max(1, min(-(-MASKED_SINGLE_BLOCKS // blocks), bound // 128, 32)) if ws is not None else 1
+        # (whole rounds of blocks over the compute units: a block of this kernel is a chain of dependent trips to memory,
+        # and a second round of a few blocks costs as much as the first)
+        nsplit = max(1, min(_compute_units(q.device) // blocks, bound // 128, 32)) if ws is not None else 1
         parts, parts_n = 0, 0
         if nsplit > 1:
             buf = ws.buffer("masked_attention.parts", (n * nh * nsplit * (dv + 2),), torch.float32)

@@ -296,6 +296,9 @@ def _close(got, ref, dtype):
     ([(200, 130), (40, 40)], 7, 1, 96, 64, 16, 0, 0, 10.0),            # seven heads on one kv head, no window
     ([(300, 200)], 4, 2, 64, 128, 32, 100, 33, 0.0),
     ([(150, 150), (500, 35)], 3, 1, 320, 256, 16, 64, 1, 0.0),
+    ([(130, 100), (40, 1)], 2, 1, 192, 128, 16, 70, 0, 0.0),
+    ([(100, 100), (300, 40), (90, 1)], 2, 2, 256, 256, 16, 64, 2, 20.0),
+    ([(140, 75)], 5, 1, 288, 256, 8, 0, 0, 0.0),
     # decoding steps at sizes that the kernel for single tokens takes in bfloat16 (1, 2 and 4 heads a block)
     ([(700, 1), (90, 1), (3, 1), (41, 1), (1, 1)], 12, 2, 128, 128, 16, 200, 4, 30.0),
     ([(700, 1), (33, 1)], 7, 1, 64, 64, 8, 0, 0, 0.0),
@@ -304,6 +307,8 @@ def _close(got, ref, dtype):
     ([(260, 1), (17, 1)], 8, 2, 192, 128, 32, 100, 40, 5.0),
     ([(3000, 1), (5, 1), (129, 1)], 4, 2, 128, 128, 16, 0, 0, 0.0),           # many splits of the keys, some of them empty
     ([(2500, 1), (300, 1)], 6, 1, 160, 128, 16, 2000, 3, 0.0),
+    ([(400, 1), (30, 1)], 3, 1, 256, 192, 16, 300, 0, 0.0),
+    ([(400, 1), (30, 1)], 4, 4, 72, 136, 16, 300, 5, 0.0),
 ])
 def test_masked_attention_against_the_plain_attention(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap):
     got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3)
