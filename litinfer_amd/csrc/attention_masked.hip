@@ -461,6 +461,20 @@ extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int
 // 8 keys at a time, the block 32, and U such rounds are in flight.  Every group of 8 lanes keeps a running
 // (maximum, sum, sums of values) per head over its keys; the groups of a wave are joined by a butterfly, the waves
 // through LDS in wave order.
+// the sum over a group of 8 neighbouring lanes, in every lane of the group, by lane moves inside the vector ALU
+// (quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror) instead of three trips through LDS
+__device__ __forceinline__ float dpp_move(float v, const int ctrl) {
+    if (ctrl == 0xB1) return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+    if (ctrl == 0x4E) return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float sum_over_8_lanes(float d) {
+    d += dpp_move(d, 0xB1);
+    d += dpp_move(d, 0x4E);
+    d += dpp_move(d, 0x141);
+    return d;
+}
+
 __device__ __forceinline__ void unpack8(const uint4 raw, float* f) {
     f[0] = __uint_as_float(raw.x << 16); f[1] = __uint_as_float(raw.x & 0xffff0000u);
     f[2] = __uint_as_float(raw.y << 16); f[3] = __uint_as_float(raw.y & 0xffff0000u);
@@ -575,10 +589,7 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
                 for (int c = 0; c < NPK; ++c)
 #pragma unroll
                     for (int e = 0; e < 8; ++e) d = fmaf(qr[hh][c][e], kf[c][e], d);      // (pieces past dk meet zeros of q)
-                d += __shfl_xor(d, 1, LI_WAVE);
-                d += __shfl_xor(d, 2, LI_WAVE);
-                d += __shfl_xor(d, 4, LI_WAVE);
-                d *= scale;
+                d = sum_over_8_lanes(d) * scale;
                 if (softcap > 0.f) d = softcap * fast_tanh(d * inv_cap);
                 sc[u][hh] = ok[u] ? d : -INFINITY;
             }

@@ -546,7 +546,8 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
         blocks = _single_blocks(n, nh, nkv, dk, dv)
         # (whole rounds of blocks over the compute units: a block of this kernel is a chain of dependent trips to memory,
         # and a second round of a few blocks costs as much as the first)
-        nsplit = max(1, min(_compute_units(q.device) // blocks, bound // 128, 32)) if ws is not None else 1
+        nsplit = max(1, min(_compute_units(q.device) * (1 if -(-dk // 64) + -(-dv // 64) > 6 else 2) // blocks,
+                             bound // 128, 32)) if ws is not None else 1
         parts, parts_n = 0, 0
         if nsplit > 1:
             buf = ws.buffer("masked_attention.parts", (n * nh * nsplit * (dv + 2),), torch.float32)
