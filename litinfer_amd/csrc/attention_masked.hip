@@ -421,6 +421,218 @@ __global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
         }
 }
 
+__global__ void masked_attention_join_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
+                                             const int* __restrict__ token_list, int nh, int dv, int nsplit);
+
+// ------------------------------------------------------------------------------------------- single tokens, MFMA
+// Decoding where a kv head serves many query heads (a compressed cache serves ALL of them): the same transposed
+// tiles with the group's HEADS as the 32 columns, one wave a (token, kv head, 32 heads, split of the keys).  Every
+// key of the token's list is visible to it, so only places past the split's end are masked.  The splits are
+// joined by `masked_attention_join_kernel`.
+template <int KS, int DT>
+__global__ __launch_bounds__(64) void masked_attention_heads_kernel(
+    const float* __restrict__ q, int q_token_stride, int q_head_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, int k_row, int v_row,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_list,
+    const int* __restrict__ seg_of_token, const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale,
+    int nsplit, float* __restrict__ parts) {
+    constexpr int DK = KS * 16, DV = DT * 32, KROW = DK + 8;
+    constexpr int NT = 64;
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[32 * KROW];       // [key place][dimension]
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[DV * MT_VS];      // [value column][key place, permuted]
+    __shared__ int rows[3][32];                                           // the cache row of each key place of three blocks in turn, -1: none
+    const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, kvh = blockIdx.y;
+    const int s = seg_of_token[t];
+    const int p0 = ctx_len[s] - q_len[s] + (t - q_start[s]);              // the token's position
+    const int p_last = p0;
+    const int lo_min = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+    const int n_first = keep_first < lo_min ? keep_first : lo_min;
+    const int n_all = n_first + (p_last - lo_min + 1);
+    const int hc = blockIdx.z / nsplit, sp = blockIdx.z % nsplit;         // the chunk of 32 heads and the split of the keys
+    const int i_begin = (int)((long)n_all * sp / nsplit), n_keys = (int)((long)n_all * (sp + 1) / nsplit);
+    const int* table = block_table + (size_t)s * max_blocks;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, ql = lane & 31, h = lane >> 5;
+    const int rep = nh / nkv;
+    const int hq = hc * 32 + ql;                                          // this lane's head within the group (a column of the tile)
+    const bool has = hq < rep;
+    const bool active = true;
+    const int head = kvh * rep + (has ? hq : 0);
+    (void)w;
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+
+    ma_frag8 qf[KS];
+    {
+        const float* qrow = q + (size_t)t * q_token_stride + (size_t)head * q_head_stride;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) {
+            const float4 a = *reinterpret_cast<const float4*>(qrow + 16 * st + 8 * h);
+            const float4 b = *reinterpret_cast<const float4*>(qrow + 16 * st + 8 * h + 4);
+            qf[st].w[0] = pack2_bf16(a.x, a.y); qf[st].w[1] = pack2_bf16(a.z, a.w);
+            qf[st].w[2] = pack2_bf16(b.x, b.y); qf[st].w[3] = pack2_bf16(b.z, b.w);
+        }
+    }
+    ma_f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    // The cache row of key place tid of the block of keys that starts at list index i0 (threads 0..31).
+    auto row_of = [&](int i0) -> int {
+        const int i = i0 + (int)threadIdx.x;
+        if (i >= n_keys) return -1;
+        const int key = visible_key(i, n_first, lo_min);
+        const int page = table[key / page_size];
+        return (page >= 0 && page < num_pages) ? (page * nkv + kvh) * page_size + key % page_size : -1;
+    };
+    constexpr int NKC = (32 * (DK / 8) + NT - 1) / NT, NVC = (32 * (DV / 8) + NT - 1) / NT;
+    uint4 kreg[NKC], vreg[NVC];
+    // a block's keys and values on their way: from memory into registers (a place without a row reads row 0 and
+    // is zeroed when it is stored) ...
+#define MT_LOAD(RB)                                                                                                   \
+    _Pragma("unroll") for (int n = 0; n < NKC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        const int kk = (i / (DK / 8)) & 31, c = i % (DK / 8), ro = rows[RB][kk];                                      \
+        kreg[n] = *reinterpret_cast<const uint4*>(kc + (size_t)(ro >= 0 ? ro : 0) * k_row + 8 * c);                   \
+    }                                                                                                                 \
+    _Pragma("unroll") for (int n = 0; n < NVC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        const int kk = i % 32, c = (i / 32) % (DV / 8), ro = rows[RB][kk];                                            \
+        vreg[n] = *reinterpret_cast<const uint4*>(vc + (size_t)(ro >= 0 ? ro : 0) * v_row + 8 * c);                   \
+    }
+    // ... and from the registers into LDS: keys as they are, values transposed and in the operand's key order
+#define MT_STORE(RB)                                                                                                  \
+    _Pragma("unroll") for (int n = 0; n < NKC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        if (i < 32 * (DK / 8)) {                                                                                      \
+            const int kk = i / (DK / 8), c = i % (DK / 8);                                                            \
+            *reinterpret_cast<uint4*>(&Ks[kk * KROW + 8 * c]) = rows[RB][kk] >= 0 ? kreg[n] : uint4{0u, 0u, 0u, 0u};  \
+        }                                                                                                             \
+    }                                                                                                                 \
+    _Pragma("unroll") for (int n = 0; n < NVC; ++n) {                                                                 \
+        const int i = threadIdx.x + NT * n;                                                                           \
+        if (i < 32 * (DV / 8)) {                                                                                      \
+            const int kk = i % 32, c = i / 32;                                                                        \
+            const uint4 raw = rows[RB][kk] >= 0 ? vreg[n] : uint4{0u, 0u, 0u, 0u};                                    \
+            const int k16 = kk & 15, rem = k16 & 7;                                                                   \
+            const int place = (kk & 16) + 8 * (rem >> 2) + 4 * (k16 >> 3) + (rem & 3);                                \
+            const uint32_t wv[4] = {raw.x, raw.y, raw.z, raw.w};                                                      \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                           \
+                Vt[(8 * c + 2 * e) * MT_VS + place] = (uint16_t)(wv[e] & 0xffffu);                                    \
+                Vt[(8 * c + 2 * e + 1) * MT_VS + place] = (uint16_t)(wv[e] >> 16);                                    \
+            }                                                                                                         \
+        }                                                                                                             \
+    }
+    const int nblk = (n_keys - i_begin + 31) / 32;
+    if (threadIdx.x < 32) {
+        rows[0][threadIdx.x] = row_of(i_begin);
+        rows[1][threadIdx.x] = row_of(i_begin + 32);
+    }
+    __syncthreads();
+    MT_LOAD(0)
+    MT_STORE(0)
+    __syncthreads();
+    // block b is in LDS; block b + 1 is asked for before b is worked on, and the rows of b + 2 before that
+    for (int b = 0; b < nblk; ++b) {
+        const int i0 = i_begin + 32 * b, rb = b % 3, rb1 = (b + 1) % 3, rb2 = (b + 2) % 3;
+        int ro2 = -1;
+        if (threadIdx.x < 32) ro2 = row_of(i0 + 64);
+        MT_LOAD(rb1)                                                      // (past the last block: its rows are -1, row 0 is read and never stored)
+        if (active) {
+            // ---- S^T = K Q^T
+            ma_f32x16 sv;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sv[r] = 0.f;
+#pragma unroll
+            for (int st = 0; st < KS; ++st) {
+                ma_frag8 kf;
+                kf.raw = *reinterpret_cast<const uint4*>(&Ks[ql * KROW + 16 * st + 8 * h]);
+                sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[st].v, sv, 0, 0, 0);
+            }
+            // ---- scale, cap, mask.  A block that every query of the tile sees whole (most are) needs no masks: its
+            // places all have rows, it lies wholly among the kept positions or wholly inside every query's window.
+            const bool whole = i0 + 31 < n_keys && __all(rows[rb][ql] >= 0);      // (every listed key is visible to the token)
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float sc = sv[r] * scale;
+                if (softcap > 0.f) sc = softcap * fast_tanh(sc * inv_cap);
+                sv[r] = sc;
+            }
+            if (!whole) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int place = 8 * (r >> 2) + 4 * h + (r & 3), i = i0 + place;
+                    const bool see = i < n_keys && rows[rb][place] >= 0;
+                    sv[r] = see ? sv[r] : -INFINITY;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sv[r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
+            const float mn = fmaxf(m, mx);
+            const float ms = (mn == -INFINITY) ? 0.f : mn;                    // a query may see no key of this block
+            const float alpha = (m == -INFINITY) ? 1.f : fast_exp(m - ms);    // (m = -inf: nothing summed yet)
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sv[r] = fast_exp(sv[r] - ms); psum += sv[r]; }
+            l = l * alpha + psum;
+            m = mn;
+            if (__any(alpha != 1.f)) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
+            }
+            ma_frag8 pf[2];
+#pragma unroll
+            for (int st = 0; st < 2; ++st)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) pf[st].w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int st = 0; st < 2; ++st) {
+                    ma_frag8 vf;
+                    vf.raw = *reinterpret_cast<const uint4*>(&Vt[(32 * dt + ql) * MT_VS + 16 * st + 8 * h]);
+                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
+                }
+        }
+        __syncthreads();                                                  // block b has been read
+        if (b + 1 < nblk) { MT_STORE(rb1) }
+        if (threadIdx.x < 32) rows[rb2][threadIdx.x] = ro2;
+        __syncthreads();
+    }
+#undef MT_LOAD
+#undef MT_STORE
+    l += __shfl_xor(l, 32, LI_WAVE);
+    if (!has) return;
+    if (nsplit == 1) {
+        const float inv = l != 0.f ? 1.0f / l : 0.f;
+        bf16_t* orow = out + ((size_t)t * nh + head) * DV;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {       // registers 4 rg .. 4 rg + 3: value columns 32 dt + 8 rg + 4 h ..
+                uint32_t* dst = reinterpret_cast<uint32_t*>(orow + 32 * dt + 8 * rg + 4 * h);
+                dst[0] = pack2_bf16(acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv);
+                dst[1] = pack2_bf16(acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv);
+            }
+    } else {                                       // this split's sums, maximum and sum of weights, for the join kernel
+        float* part = parts + (((size_t)blockIdx.x * nh + head) * nsplit + sp) * (DV + 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) part[32 * dt + 8 * rg + 4 * h + e] = acc[dt][4 * rg + e];
+        if (h == 0) { part[DV] = m; part[DV + 1] = l; }
+    }
+}
+
 // 1 if the tile kernel takes these sizes (bfloat16 cache and output)
 extern "C" int li_masked_attention_tiles_takes(int dk, int dv) {
 #define MT_HAS(K, V) if (dk == K && dv == V) return 1;
@@ -451,6 +663,36 @@ extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int
     MT_GO(64, 64) MT_GO(128, 128) MT_GO(128, 64) MT_GO(64, 128) MT_GO(96, 64) MT_GO(160, 128) MT_GO(192, 128)
     MT_GO(256, 256) MT_GO(320, 256) MT_GO(288, 256)
 #undef MT_GO
+    return LI_ERR_SIZE;
+}
+
+
+extern "C" int li_masked_attention_heads(const float* q, int q_token_stride, int q_head_stride, void* out, const void* kc,
+                                         const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
+                                         const int* token_list, int n_tokens, const int* seg_of_token, const int* q_start,
+                                         const int* q_len, const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size,
+                                         int num_pages, int window, int keep_first, float softcap, float scale, int nsplit,
+                                         float* parts, long parts_floats, hipStream_t stream) {
+    if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
+        window < 0 || keep_first < 0 || max_blocks <= 0 || k_row % 8 || v_row % 8 || q_token_stride % 4 || q_head_stride % 4 ||
+        ((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) % 16 || (uintptr_t)out % 8 || !li_masked_attention_tiles_takes(dk, dv) ||
+        nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!parts || parts_floats < (long)n_tokens * nh * nsplit * (dv + 2))))
+        return LI_ERR_SIZE;
+    const int rep = nh / nkv;
+    const dim3 grid(n_tokens, nkv, ((rep + 31) / 32) * nsplit);
+#define MH_GO(K, V)                                                                                                        \
+    if (dk == K && dv == V) {                                                                                              \
+        masked_attention_heads_kernel<K / 16, V / 32><<<grid, 64, 0, stream>>>(                                            \
+            q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
+            max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, \
+            softcap, scale, nsplit, parts);                                                                                \
+        if (nsplit > 1)                                                                                                    \
+            masked_attention_join_kernel<<<dim3(n_tokens, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, token_list, nh, dv, nsplit); \
+        return li_launch_status();                                                                                         \
+    }
+    MH_GO(64, 64) MH_GO(128, 128) MH_GO(128, 64) MH_GO(64, 128) MH_GO(96, 64) MH_GO(160, 128) MH_GO(192, 128)
+    MH_GO(256, 256) MH_GO(320, 256) MH_GO(288, 256)
+#undef MH_GO
     return LI_ERR_SIZE;
 }
 

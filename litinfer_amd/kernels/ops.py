@@ -48,6 +48,7 @@ _SIGNATURES = {
     "attention_masked": {
         "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I],
         "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
+        "li_masked_attention_heads": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
         "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F],
         "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I],
     },
@@ -539,6 +540,22 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
 
     def singles(token_list, n):
         # single tokens in bfloat16, at the sizes it has: rows spread over lanes, a row read once for a group's heads
+        if (fast and nh // nkv >= MASKED_HEADS_MIN and n * (nh // nkv) >= MASKED_HEADS_MIN_WORK and masked_tiles_take(dk, dv)
+                and ws is not None):
+            # many query heads on one kv head (a compressed cache: all of them): the heads are the columns of
+            # matrix-core tiles, one wave a (token, kv head, 32 heads, split of the keys)
+            blocks = n * nkv * -(-(nh // nkv) // 32)
+            nsplit = max(1, min(3 * _compute_units(q.device) // blocks, bound // 64, 32))
+            parts, parts_n = 0, 0
+            if nsplit > 1:
+                buf = ws.buffer("masked_attention.parts", (n * nh * nsplit * (dv + 2),), torch.float32)
+                parts, parts_n = buf.data_ptr(), buf.numel()
+            return _run("attention_masked", "li_masked_attention_heads", q.data_ptr(), int(q_token_stride),
+                        int(q_head_stride), out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3],
+                        meta.block_table.data_ptr(), meta.max_blocks, 0 if token_list is None else token_list.data_ptr(), n,
+                        meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
+                        nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0),
+                        float(scale), nsplit, parts, parts_n)
         if not (fast and masked_single_takes(dk, dv)):
             return general(token_list, n)
         # few blocks against many keys: the keys are cut into splits, each a block of its own, and joined by a second
@@ -573,6 +590,11 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
     general(None, t)
 
 
+MASKED_HEADS_MIN = 8          # query heads a kv head from which single tokens take the matrix-core kernel (8 of its 32 columns)
+# ... and the (token, head) pairs of a kv head from which it is the faster one: with fewer, the vector kernel's many small
+# blocks finish sooner than a wave that stages every block of keys through LDS by itself (measured at 8 and 64 requests
+# of 12 and 28 heads: 0.95 against 1.09 ms and 1.32 against 1.50 ms a step of 12 heads, 2.28 against 2.22 ms at 64 x 28)
+MASKED_HEADS_MIN_WORK = 1024
 MASKED_TILE_ROWS = 32         # queries of one request that a block of the matrix-core kernel takes
 
 

@@ -210,7 +210,7 @@ def _meta(seg_specs, page, tables):
 
 
 def _masked_case(dtype, seg_specs, nh, nkv, dk, dv, page, window, keep_first, softcap, seed, standout=None,
-                 shared_rows=False, return_values=False):
+                 shared_rows=False, return_values=False, heads_kernel=False):
     """Random queries, keys and values for segments (context, queries); pages in shuffled order with garbage
     in every slot that no key owns (and -1 in the table where a windowed cache would have given a page back).
     `standout` = (key position, query row): that key's score is made to win by e^12.  `shared_rows`: values are
@@ -259,8 +259,14 @@ def _masked_case(dtype, seg_specs, nh, nkv, dk, dv, page, window, keep_first, so
     kd = kc.to(DEV)
     vd = kd if shared_rows else vc.to(DEV)
     from litinfer_amd.engine.workspace import Workspace
-    ops.masked_attention(qd, nh * dk, dk, out, kd, vd, meta, nh, nkv, dk, dv, page, window, keep_first, softcap, scale,
-                         ws=Workspace(DEV))
+    was = ops.MASKED_HEADS_MIN_WORK
+    if heads_kernel:                                     # single tokens on the matrix cores whatever their number
+        ops.MASKED_HEADS_MIN_WORK = 0
+    try:
+        ops.masked_attention(qd, nh * dk, dk, out, kd, vd, meta, nh, nkv, dk, dv, page, window, keep_first, softcap, scale,
+                             ws=Workspace(DEV))
+    finally:
+        ops.MASKED_HEADS_MIN_WORK = was
     refs, o = [], 0
     rep = nh // nkv
     for s, (c, ql) in enumerate(seg_specs):
@@ -309,10 +315,17 @@ def _close(got, ref, dtype):
     ([(2500, 1), (300, 1)], 6, 1, 160, 128, 16, 2000, 3, 0.0),
     ([(400, 1), (30, 1)], 3, 1, 256, 192, 16, 300, 0, 0.0),
     ([(400, 1), (30, 1)], 4, 4, 72, 136, 16, 300, 5, 0.0),
+    # many heads on one kv head: single tokens on the matrix cores, the heads as a tile's columns
+    ([(700, 1), (90, 1), (3, 1), (41, 1), (1, 1)], 12, 1, 128, 128, 16, 200, 4, 30.0),
+    ([(1500, 1), (100, 1), (64, 1)], 40, 1, 320, 256, 16, 1024, 0, 0.0),            # two chunks of 32 heads
+    ([(300, 1), (33, 1), (200, 60)], 18, 2, 64, 64, 8, 0, 0, 0.0),                 # beside a portion
 ])
 def test_masked_attention_against_the_plain_attention(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap):
     got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3)
     _close(got, ref, dtype)
+    if nh // nkv >= 8:
+        got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3, heads_kernel=True)
+        _close(got, ref, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -323,6 +336,10 @@ def test_values_that_are_the_first_columns_of_the_keys_rows(dtype):
     _close(got, ref, dtype)
     got, ref = _masked_case(dtype, [(400, 1), (77, 1), (1, 1)], 4, 1, 160, 128, 16, 90, 0, 0.0, seed=6, shared_rows=True)
     _close(got, ref, dtype)
+    for heads_kernel in (False, True):
+        got, ref = _masked_case(dtype, [(900, 1), (77, 1), (1, 1)], 10, 1, 160, 128, 16, 500, 0, 0.0, seed=7, shared_rows=True,
+                                heads_kernel=heads_kernel)
+        _close(got, ref, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
