@@ -540,8 +540,7 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
 
     def singles(token_list, n):
         # single tokens in bfloat16, at the sizes it has: rows spread over lanes, a row read once for a group's heads
-        if (fast and nh // nkv >= MASKED_HEADS_MIN and n * (nh // nkv) >= MASKED_HEADS_MIN_WORK and masked_tiles_take(dk, dv)
-                and ws is not None):
+        if fast and ws is not None and masked_tiles_take(dk, dv) and _heads_kernel_pays(n, nh // nkv, dk, dv):
             # many query heads on one kv head (a compressed cache: all of them): the heads are the columns of
             # matrix-core tiles, one wave a (token, kv head, 32 heads, split of the keys)
             blocks = n * nkv * -(-(nh // nkv) // 32)
@@ -590,11 +589,24 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
     general(None, t)
 
 
-MASKED_HEADS_MIN = 8          # query heads a kv head from which single tokens take the matrix-core kernel (8 of its 32 columns)
-# ... and the (token, head) pairs of a kv head from which it is the faster one: with fewer, the vector kernel's many small
-# blocks finish sooner than a wave that stages every block of keys through LDS by itself (measured at 8 and 64 requests
-# of 12 and 28 heads: 0.95 against 1.09 ms and 1.32 against 1.50 ms a step of 12 heads, 2.28 against 2.22 ms at 64 x 28)
+# Single tokens on the matrix cores (the heads of a kv head as a tile's columns) or on the vector ALU.  Measured on
+# 8 / 64 / 256 requests of 1,028 visible keys (us a call, vector against matrix cores): rows of 128 + 128 columns,
+# 28 heads on 4 kv heads 46/20, 84/49, 324/127; 12 on 2: 19/19, 36/33, 152/107; rows of 320 columns shared by keys and
+# values (a compressed cache), 28 heads: 28/38, 144/112, 494/396; 12 heads: 21/36, 74/107, 225/381 (there one wave
+# stages 36 KB a block of keys by itself, which sets its time whatever the heads).
+# One and two requests: 28 on 4: 25/24, 24/24; 12 on 2: 19/23, 18/23; the long rows 20/40.
+MASKED_HEADS_MIN = 4          # query heads a kv head from which rows of up to 384 columns (keys + values) take the matrix cores,
+MASKED_HEADS_MIN_PAIRS = 48   # for at least so many (token, head) pairs a kv head
+MASKED_HEADS_MIN_LONG = 24    # ... and from which longer rows do, for at least MASKED_HEADS_MIN_WORK (token, head) pairs a kv head
 MASKED_HEADS_MIN_WORK = 1024
+
+
+def _heads_kernel_pays(n: int, rep: int, dk: int, dv: int) -> bool:
+    if dk + dv <= 384:
+        return rep >= MASKED_HEADS_MIN and n * rep >= MASKED_HEADS_MIN_PAIRS
+    return rep >= MASKED_HEADS_MIN_LONG and n * rep >= MASKED_HEADS_MIN_WORK
+
+
 MASKED_TILE_ROWS = 32         # queries of one request that a block of the matrix-core kernel takes
 
 

@@ -210,7 +210,7 @@ def _meta(seg_specs, page, tables):
 
 
 def _masked_case(dtype, seg_specs, nh, nkv, dk, dv, page, window, keep_first, softcap, seed, standout=None,
-                 shared_rows=False, return_values=False, heads_kernel=False):
+                 shared_rows=False, return_values=False, heads_kernel=None):
     """Random queries, keys and values for segments (context, queries); pages in shuffled order with garbage
     in every slot that no key owns (and -1 in the table where a windowed cache would have given a page back).
     `standout` = (key position, query row): that key's score is made to win by e^12.  `shared_rows`: values are
@@ -259,14 +259,14 @@ def _masked_case(dtype, seg_specs, nh, nkv, dk, dv, page, window, keep_first, so
     kd = kc.to(DEV)
     vd = kd if shared_rows else vc.to(DEV)
     from litinfer_amd.engine.workspace import Workspace
-    was = ops.MASKED_HEADS_MIN_WORK
-    if heads_kernel:                                     # single tokens on the matrix cores whatever their number
-        ops.MASKED_HEADS_MIN_WORK = 0
+    was = ops._heads_kernel_pays
+    if heads_kernel is not None:                         # single tokens on the matrix cores, or not, whatever their number
+        ops._heads_kernel_pays = lambda *a: bool(heads_kernel)
     try:
         ops.masked_attention(qd, nh * dk, dk, out, kd, vd, meta, nh, nkv, dk, dv, page, window, keep_first, softcap, scale,
                              ws=Workspace(DEV))
     finally:
-        ops.MASKED_HEADS_MIN_WORK = was
+        ops._heads_kernel_pays = was
     refs, o = [], 0
     rep = nh // nkv
     for s, (c, ql) in enumerate(seg_specs):
@@ -323,8 +323,8 @@ def _close(got, ref, dtype):
 def test_masked_attention_against_the_plain_attention(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap):
     got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3)
     _close(got, ref, dtype)
-    if nh // nkv >= 8:
-        got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3, heads_kernel=True)
+    for heads_kernel in (False, True):                   # single tokens on the vector ALU and on the matrix cores
+        got, ref = _masked_case(dtype, segs, nh, nkv, dk, dv, page, window, keep, cap, seed=3, heads_kernel=heads_kernel)
         _close(got, ref, dtype)
 
 
