@@ -227,15 +227,15 @@ union ma_frag8 { uint4 raw; uint32_t w[4]; ma_bf16x8 v; };
 #define MT_WAVES 4
 #define MT_VS 40                    // row stride of the transposed values: 32 key places and a pad that spreads the banks
 
-template <int KS, int DT>           // KS = dk / 16, DT = dv / 32
-__global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
+template <int KS, int DT, int NW>   // KS = dk / 16, DT = dv / 32, NW waves = heads of the kv head a block
+__global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
     const float* __restrict__ q, int q_token_stride, int q_head_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, int k_row, int v_row,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
     int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale) {
     constexpr int DK = KS * 16, DV = DT * 32, KROW = DK + 8;
-    constexpr int NT = MT_WAVES * 64;
+    constexpr int NT = NW * 64;
     __shared__ __attribute__((aligned(16))) uint16_t Ks[32 * KROW];       // [key place][dimension]
     __shared__ __attribute__((aligned(16))) uint16_t Vt[DV * MT_VS];      // [value column][key place, permuted]
     __shared__ int rows[3][32];                                           // the cache row of each key place of three blocks in turn, -1: none
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(MT_WAVES * 64) void masked_attention_tile_kernel(
     const int* table = block_table + (size_t)s * max_blocks;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, ql = lane & 31, h = lane >> 5;
     const int rep = nh / nkv;
-    const int hh = blockIdx.z * MT_WAVES + w;                             // this wave's head within the group
+    const int hh = blockIdx.z * NW + w;                             // this wave's head within the group
     const bool active = hh < rep;
     const int head = kvh * rep + (active ? hh : 0);
     const int pq = p0 + ql;                                               // this lane's query (ql >= ntok: none)
@@ -652,12 +652,20 @@ extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int
         ((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) % 16 || (uintptr_t)out % 8 || !li_masked_attention_tiles_takes(dk, dv))
         return LI_ERR_SIZE;
     const int rep = nh / nkv;
-    const dim3 grid(num_tiles, nkv, (rep + MT_WAVES - 1) / MT_WAVES);
+    // five to eight heads a kv head: one block of eight waves (one staging of every block of keys for all of them)
+    // rather than blocks of four and of one to four; more heads: whichever leaves fewer waves idle
+    const int nw = (rep > 4 && (rep <= 8 || rep % 8 == 0 || rep % 8 > 4)) ? 8 : 4;
+    const dim3 grid(num_tiles, nkv, (rep + nw - 1) / nw);
 #define MT_GO(K, V)                                                                                                        \
     if (dk == K && dv == V) {                                                                                              \
-        masked_attention_tile_kernel<K / 16, V / 32><<<grid, MT_WAVES * 64, 0, stream>>>(                                  \
-            q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
-            max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale); \
+        if (nw == 8)                                                                                                       \
+            masked_attention_tile_kernel<K / 16, V / 32, 8><<<grid, 512, 0, stream>>>(                                     \
+                q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
+                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale); \
+        else                                                                                                               \
+            masked_attention_tile_kernel<K / 16, V / 32, 4><<<grid, 256, 0, stream>>>(                                     \
+                q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
+                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale); \
         return li_launch_status();                                                                                         \
     }
     MT_GO(64, 64) MT_GO(128, 128) MT_GO(128, 64) MT_GO(64, 128) MT_GO(96, 64) MT_GO(160, 128) MT_GO(192, 128)
