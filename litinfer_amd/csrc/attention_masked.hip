@@ -233,12 +233,13 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, int k_row, int v_row,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
-    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale) {
+    int nh, int nkv, int page_size, int num_pages, int window, int keep_first, float softcap, float scale,
+    int nsplit, float* __restrict__ parts) {
     constexpr int DK = KS * 16, DV = DT * 32, KROW = DK + 8;
     constexpr int NT = NW * 64;
     __shared__ __attribute__((aligned(16))) uint16_t Ks[32 * KROW];       // [key place][dimension]
     __shared__ __attribute__((aligned(16))) uint16_t Vt[DV * MT_VS];      // [value column][key place, permuted]
-    __shared__ int rows[3][32];                                           // the cache row of each key place of three blocks in turn, -1: none
+    __shared__ int rows[4][32];                                           // the cache row of each key place of four blocks in turn, -1: none
     const int tile = blockIdx.x, kvh = blockIdx.y;
     const int s = tiles[4 * tile], t0 = tiles[4 * tile + 1], ntok = tiles[4 * tile + 2];
     const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);             // position of the tile's first query
@@ -249,7 +250,8 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
     const int* table = block_table + (size_t)s * max_blocks;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, ql = lane & 31, h = lane >> 5;
     const int rep = nh / nkv;
-    const int hh = blockIdx.z * NW + w;                             // this wave's head within the group
+    const int sp = blockIdx.z % nsplit;                                    // this block's share of the tile's blocks of keys
+    const int hh = (blockIdx.z / nsplit) * NW + w;                             // this wave's head within the group
     const bool active = hh < rep;
     const int head = kvh * rep + (active ? hh : 0);
     const int pq = p0 + ql;                                               // this lane's query (ql >= ntok: none)
@@ -284,10 +286,10 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
         return (page >= 0 && page < num_pages) ? (page * nkv + kvh) * page_size + key % page_size : -1;
     };
     constexpr int NKC = (32 * (DK / 8) + NT - 1) / NT, NVC = (32 * (DV / 8) + NT - 1) / NT;
-    uint4 kreg[NKC], vreg[NVC];
+    uint4 kregA[NKC], vregA[NVC], kregB[NKC], vregB[NVC];           // two blocks of keys on their way at a time
     // a block's keys and values on their way: from memory into registers (a place without a row reads row 0 and
     // is zeroed when it is stored) ...
-#define MT_LOAD(RB)                                                                                                   \
+#define MT_LOAD(RB, kreg, vreg)                                                                                                   \
     _Pragma("unroll") for (int n = 0; n < NKC; ++n) {                                                                 \
         const int i = threadIdx.x + NT * n;                                                                           \
         const int kk = (i / (DK / 8)) & 31, c = i % (DK / 8), ro = rows[RB][kk];                                      \
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
         vreg[n] = *reinterpret_cast<const uint4*>(vc + (size_t)(ro >= 0 ? ro : 0) * v_row + 8 * c);                   \
     }
     // ... and from the registers into LDS: keys as they are, values transposed and in the operand's key order
-#define MT_STORE(RB)                                                                                                  \
+#define MT_STORE(RB, kreg, vreg)                                                                                                  \
     _Pragma("unroll") for (int n = 0; n < NKC; ++n) {                                                                 \
         const int i = threadIdx.x + NT * n;                                                                           \
         if (i < 32 * (DK / 8)) {                                                                                      \
@@ -321,21 +323,30 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
             }                                                                                                         \
         }                                                                                                             \
     }
-    const int nblk = (n_keys + 31) / 32;
+    const int nblk_all = (n_keys + 31) / 32;
+    const int b_begin = (int)((long)nblk_all * sp / nsplit), nblk = (int)((long)nblk_all * (sp + 1) / nsplit) - b_begin;
     if (threadIdx.x < 32) {
-        rows[0][threadIdx.x] = row_of(0);
-        rows[1][threadIdx.x] = row_of(32);
+        rows[0][threadIdx.x] = row_of(32 * b_begin);
+        rows[1][threadIdx.x] = row_of(32 * b_begin + 32);
+        rows[2][threadIdx.x] = row_of(32 * b_begin + 64);
     }
     __syncthreads();
-    MT_LOAD(0)
-    MT_STORE(0)
+    MT_LOAD(0, kregA, vregA)
+    MT_LOAD(1, kregB, vregB)
+    MT_STORE(0, kregA, vregA)
     __syncthreads();
-    // block b is in LDS; block b + 1 is asked for before b is worked on, and the rows of b + 2 before that
-    for (int b = 0; b < nblk; ++b) {
-        const int i0 = 32 * b, rb = b % 3, rb1 = (b + 1) % 3, rb2 = (b + 2) % 3;
-        int ro2 = -1;
-        if (threadIdx.x < 32) ro2 = row_of(i0 + 64);
-        MT_LOAD(rb1)                                                      // (past the last block: its rows are -1, row 0 is read and never stored)
+    // Block b is in LDS and block b + 1 in registers; block b + 2 is asked for before b is worked on, and the rows of
+    // b + 3 before that: a trip to memory has two turns' time.  Two turns a trip, so that the registers of a turn are
+    // a constant of the code.
+    for (int b2 = 0; b2 < nblk; b2 += 2) {
+#pragma unroll
+      for (int turn = 0; turn < 2; ++turn) {
+        const int b = b2 + turn;
+        if (b >= nblk) break;
+        const int i0 = 32 * (b_begin + b), rb = b & 3, rb1 = (b + 1) & 3, rb2 = (b + 2) & 3, rb3 = (b + 3) & 3;
+        int ro3 = -1;
+        if (threadIdx.x < 32) ro3 = row_of(i0 + 96);
+        if (turn == 0) { MT_LOAD(rb2, kregA, vregA) } else { MT_LOAD(rb2, kregB, vregB) }     // (past the last block: rows -1, row 0 is read and never stored)
         if (active) {
             // ---- S^T = K Q^T
             ma_f32x16 sv;
@@ -400,15 +411,32 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
                 }
         }
         __syncthreads();                                                  // block b has been read
-        if (b + 1 < nblk) { MT_STORE(rb1) }
-        if (threadIdx.x < 32) rows[rb2][threadIdx.x] = ro2;
+        if (b + 1 < nblk) {
+            if (turn == 0) { MT_STORE(rb1, kregB, vregB) } else { MT_STORE(rb1, kregA, vregA) }
+        }
+        if (threadIdx.x < 32) rows[rb3][threadIdx.x] = ro3;
         __syncthreads();
+      }
     }
 #undef MT_LOAD
 #undef MT_STORE
     if (!active) return;
     l += __shfl_xor(l, 32, LI_WAVE);
     if (ql >= ntok) return;
+    if (nsplit > 1) {                              // this split's sums, maximum and sum of weights, for the join kernel
+        float* part = parts + (((size_t)(t0 + ql) * nh + head) * nsplit + sp) * (DV + 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg)
+            {                                      // (a part starts on 8 bytes)
+                float2* dst = reinterpret_cast<float2*>(part + 32 * dt + 8 * rg + 4 * h);
+                dst[0] = float2{acc[dt][4 * rg], acc[dt][4 * rg + 1]};
+                dst[1] = float2{acc[dt][4 * rg + 2], acc[dt][4 * rg + 3]};
+            }
+        if (h == 0) { part[DV] = m; part[DV + 1] = l; }
+        return;
+    }
     const float inv = l != 0.f ? 1.0f / l : 0.f;
     bf16_t* orow = out + ((size_t)(t0 + ql) * nh + head) * DV;
 #pragma unroll
@@ -422,7 +450,7 @@ __global__ __launch_bounds__(NW * 64) void masked_attention_tile_kernel(
 }
 
 __global__ void masked_attention_join_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
-                                             const int* __restrict__ token_list, int nh, int dv, int nsplit);
+                                             const int* __restrict__ token_list, int nh, int dv, int nsplit, int by_token = 0);
 
 // ------------------------------------------------------------------------------------------- single tokens, MFMA
 // Decoding where a kv head serves many query heads (a compressed cache serves ALL of them): the same transposed
@@ -646,26 +674,34 @@ extern "C" int li_masked_attention_tiles(const float* q, int q_token_stride, int
                                          const void* vc, int k_row, int v_row, const int* block_table, int max_blocks,
                                          const int* tiles, int num_tiles, const int* q_start, const int* q_len,
                                          const int* ctx_len, int nh, int nkv, int dk, int dv, int page_size, int num_pages,
-                                         int window, int keep_first, float softcap, float scale, hipStream_t stream) {
+                                         int window, int keep_first, float softcap, float scale, int nsplit, float* parts,
+                                         long parts_floats, const int* multi_tokens, int num_multi, int num_tokens,
+                                         hipStream_t stream) {
     if (num_tiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || dk > k_row || dv > v_row || page_size <= 0 ||
         window < 0 || keep_first < 0 || max_blocks <= 0 || k_row % 8 || v_row % 8 || q_token_stride % 4 || q_head_stride % 4 ||
-        ((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) % 16 || (uintptr_t)out % 8 || !li_masked_attention_tiles_takes(dk, dv))
+        ((uintptr_t)q | (uintptr_t)kc | (uintptr_t)vc) % 16 || (uintptr_t)out % 8 || !li_masked_attention_tiles_takes(dk, dv) ||
+        nsplit < 1 || nsplit > 16 || num_multi <= 0 ||
+        (nsplit > 1 && (!parts || (uintptr_t)parts % 8 || parts_floats < (long)num_tokens * nh * nsplit * (dv + 2))))
         return LI_ERR_SIZE;
     const int rep = nh / nkv;
     // five to eight heads a kv head: one block of eight waves (one staging of every block of keys for all of them)
     // rather than blocks of four and of one to four; more heads: whichever leaves fewer waves idle
     const int nw = (rep > 4 && (rep <= 8 || rep % 8 == 0 || rep % 8 > 4)) ? 8 : 4;
-    const dim3 grid(num_tiles, nkv, (rep + nw - 1) / nw);
+    const dim3 grid(num_tiles, nkv, ((rep + nw - 1) / nw) * nsplit);
 #define MT_GO(K, V)                                                                                                        \
     if (dk == K && dv == V) {                                                                                              \
         if (nw == 8)                                                                                                       \
             masked_attention_tile_kernel<K / 16, V / 32, 8><<<grid, 512, 0, stream>>>(                                     \
                 q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
-                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale); \
+                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale, \
+                nsplit, parts);                                                                                            \
         else                                                                                                               \
             masked_attention_tile_kernel<K / 16, V / 32, 4><<<grid, 256, 0, stream>>>(                                     \
                 q, q_token_stride, q_head_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, k_row, v_row, block_table, \
-                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale); \
+                max_blocks, tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, keep_first, softcap, scale, \
+                nsplit, parts);                                                                                            \
+        if (nsplit > 1)                                                                                                    \
+            masked_attention_join_kernel<<<dim3(num_multi, nh), dv >= 256 ? 256 : 128, 0, stream>>>(parts, (bf16_t*)out, multi_tokens, nh, dv, nsplit, 1); \
         return li_launch_status();                                                                                         \
     }
     MT_GO(64, 64) MT_GO(128, 128) MT_GO(128, 64) MT_GO(64, 128) MT_GO(96, 64) MT_GO(160, 128) MT_GO(192, 128)
@@ -941,10 +977,11 @@ __global__ __launch_bounds__(256) void masked_attention_single_kernel(
 }
 
 // joins the splits of every (token, head) in split order: a block a (token, head)
+// (the parts of a token lie at its place in the list, or, with by_token, at its own number)
 __global__ void masked_attention_join_kernel(const float* __restrict__ parts, bf16_t* __restrict__ out,
-                                             const int* __restrict__ token_list, int nh, int dv, int nsplit) {
+                                             const int* __restrict__ token_list, int nh, int dv, int nsplit, int by_token) {
     const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, head = blockIdx.y;
-    const float* base = parts + ((size_t)blockIdx.x * nh + head) * nsplit * (dv + 2);
+    const float* base = parts + ((size_t)(by_token ? t : (int)blockIdx.x) * nh + head) * nsplit * (dv + 2);
     float mm = -INFINITY;
     for (int x = 0; x < nsplit; ++x) mm = fmaxf(mm, base[(size_t)x * (dv + 2) + dv]);
     for (int d = threadIdx.x; d < dv; d += blockDim.x) {

@@ -49,7 +49,7 @@ _SIGNATURES = {
         "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I],
         "li_masked_attention_single": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
         "li_masked_attention_heads": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L],
-        "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F],
+        "li_masked_attention_tiles": [P, I, I, P, P, P, I, I, P, I, P, I, P, P, P, I, I, I, I, I, I, I, I, F, F, I, P, L, P, I, I],
         "li_headwise_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I],
     },
     "gemm": {
@@ -579,10 +579,24 @@ def masked_attention(q: torch.Tensor, q_token_stride: int, q_head_stride: int, o
     # portions of prompts in bfloat16, at the sizes it has: tiles of queries on the matrix cores
     if (fast and meta.tiles is not None and meta.num_tiles and meta.tile_rows == MASKED_TILE_ROWS and masked_tiles_take(dk, dv)
             and meta.num_single + meta.num_multi == t):
+        # few tiles (one prompt of a model with few kv heads): a wave's own chain of matrix products and softmax sets
+        # the time of a block of keys, so the waves must fill the chip: a tile's blocks of keys are cut into splits,
+        # each a block of its own, and joined by the kernel that joins single tokens' splits
+        rep = nh // nkv
+        nw = 8 if rep > 4 and (rep <= 8 or rep % 8 == 0 or rep % 8 > 4) else 4
+        waves = meta.num_tiles * nkv * -(-rep // nw) * nw
+        slots = (8 if dk + dv <= 384 else 4) * _compute_units(q.device)      # waves the chip holds of this kernel (its registers)
+        nsplit = max(1, min(slots // waves, bound // 128, 4)) if ws is not None else 1
+        n_multi = meta.num_multi or t
+        parts, parts_n = 0, 0
+        if nsplit > 1:
+            buf = ws.buffer("masked_attention.parts", (t * nh * nsplit * (dv + 2),), torch.float32)
+            parts, parts_n = buf.data_ptr(), buf.numel()
         _run("attention_masked", "li_masked_attention_tiles", q.data_ptr(), int(q_token_stride), int(q_head_stride),
              out.data_ptr(), k.data_ptr(), v.data_ptr(), k.shape[3], v.shape[3], meta.block_table.data_ptr(), meta.max_blocks,
              meta.tiles.data_ptr(), meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
-             nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale))
+             nh, nkv, dk, dv, page_size, k.shape[0], int(window), int(keep_first), float(softcap or 0.0), float(scale),
+             nsplit, parts, parts_n, 0 if meta.multi_tokens is None else meta.multi_tokens.data_ptr(), n_multi, t)
         if meta.num_single:
             singles(meta.single_tokens, meta.num_single)       # (a list is there: the batch has tokens of both kinds)
         return

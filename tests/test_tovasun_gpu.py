@@ -305,6 +305,8 @@ def _close(got, ref, dtype):
     ([(130, 100), (40, 1)], 2, 1, 192, 128, 16, 70, 0, 0.0),
     ([(100, 100), (300, 40), (90, 1)], 2, 2, 256, 256, 16, 64, 2, 20.0),
     ([(140, 75)], 5, 1, 288, 256, 8, 0, 0, 0.0),
+    ([(700, 300), (64, 1), (400, 33)], 4, 2, 64, 64, 16, 0, 0, 0.0),            # few tiles against many keys: splits of a tile's keys
+    ([(900, 200), (300, 1)], 6, 1, 128, 128, 16, 512, 7, 25.0),
     # decoding steps at sizes that the kernel for single tokens takes in bfloat16 (1, 2 and 4 heads a block)
     ([(700, 1), (90, 1), (3, 1), (41, 1), (1, 1)], 12, 2, 128, 128, 16, 200, 4, 30.0),
     ([(700, 1), (33, 1)], 7, 1, 64, 64, 8, 0, 0, 0.0),
