@@ -12,6 +12,10 @@ from .tovasun import TovasunConfig, tovasun_model_spec
 
 register_architecture("Tovasun", TovasunConfig.from_dict, tovasun_model_spec, aliases=("tovasun",))
 
-__all__ = ["TovasunConfig", "tovasun_model_spec", "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "Architecture", "architecture_name",
+from .sogenex import SogenexConfig, sogenex_model_spec
+
+register_architecture("Sogenex", SogenexConfig.from_dict, sogenex_model_spec, aliases=("sogenex",))
+
+__all__ = ["TovasunConfig", "tovasun_model_spec", "SogenexConfig", "sogenex_model_spec", "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "Architecture", "architecture_name",
            "load_config", "lookup", "read_config_json", "register_architecture",
            "registered_architectures", "ConfigError", "Qwen2Config", "qwen2_model_spec"]

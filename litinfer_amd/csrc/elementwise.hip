@@ -712,3 +712,112 @@ extern "C" int li_latent_norm_pairs_store(const float* qd, int row_stride, int n
     else return LI_ERR_DTYPE;
     return li_launch_status();
 }
+
+// ------------------------------------------------------------------------------ sinusoidal position vector
+// x[t, 2i] += sin(p f_i), x[t, 2i + 1] += cos(p f_i) with p = positions[t] and f the table of frequencies
+// (worked out by the caller, one per pair of columns); the angle is float(p) * f_i in float32.
+__global__ void sinusoid_add_kernel(float* __restrict__ x, const int* __restrict__ positions, const float* __restrict__ freq, int H) {
+    const int t = blockIdx.x;
+    const float p = (float)positions[t];
+    float* row = x + (size_t)t * H;
+    for (int i = threadIdx.x; 2 * i < H; i += blockDim.x) {
+        const float a = p * freq[i];
+        row[2 * i] += sinf(a);
+        if (2 * i + 1 < H) row[2 * i + 1] += cosf(a);
+    }
+}
+
+extern "C" int li_sinusoid_add(float* x, const int* positions, const float* freq, int T, int H, hipStream_t stream) {
+    if (T <= 0 || H <= 0) return LI_ERR_SIZE;
+    sinusoid_add_kernel<<<T, 256, 0, stream>>>(x, positions, freq, H);
+    return li_launch_status();
+}
+
+// ------------------------------------------------------------------------------ scaled and capped logits
+// v <- v * scale, then, where cap > 0, cap * tanh(v / cap)
+__global__ void scale_softcap_kernel(float* __restrict__ x, long n, float scale, float cap) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float v = x[i] * scale;
+        x[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+    }
+}
+
+extern "C" int li_scale_softcap(float* x, long n, float scale, float cap, hipStream_t stream) {
+    if (n <= 0 || cap < 0.f) return LI_ERR_SIZE;
+    scale_softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, n, scale, cap);
+    return li_launch_status();
+}
+
+// ------------------------------------------------------------------------------ columns of rows into pages
+// Up to three runs of columns of a float32 row (run r: `heads[r]` heads of `dim[r]` columns from column col[r] on) go to
+// the token's slot in three paged tensors [pages, heads, page_size, dim].
+struct PagedRuns { int col[3]; int heads[3]; int dim[3]; void* dst[3]; };
+
+template <typename T>
+__global__ void paged_store_kernel(const float* __restrict__ src, long stride, PagedRuns runs, const int* __restrict__ slot_map,
+                                   int page_size) {
+    const int t = blockIdx.x;
+    const int slot = slot_map[t], page = slot / page_size, off = slot % page_size;
+    const float* row = src + (size_t)t * stride;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        const int nh = runs.heads[r], d = runs.dim[r];
+        T* dst = (T*)runs.dst[r];
+        for (int u = threadIdx.x; u < nh * d; u += blockDim.x) {
+            const int h = u / d, j = u % d;
+            store_from_float(dst + ((size_t)(page * nh + h) * page_size + off) * d + j, row[runs.col[r] + u]);
+        }
+    }
+}
+
+extern "C" int li_paged_store(const float* src, long stride, int col0, int heads0, int dim0, void* dst0, int col1, int heads1,
+                              int dim1, void* dst1, int col2, int heads2, int dim2, void* dst2, int cache_dtype,
+                              const int* slot_map, int page_size, int T, hipStream_t stream) {
+    if (T <= 0 || page_size <= 0 || heads0 < 0 || heads1 < 0 || heads2 < 0 || dim0 < 0 || dim1 < 0 || dim2 < 0) return LI_ERR_SIZE;
+    PagedRuns runs{{col0, col1, col2}, {heads0, heads1, heads2}, {dim0, dim1, dim2}, {dst0, dst1, dst2}};
+    for (int r = 0; r < 3; ++r)
+        if (runs.heads[r] && (runs.col[r] < 0 || runs.col[r] + (long)runs.heads[r] * runs.dim[r] > stride || !runs.dst[r])) return LI_ERR_SIZE;
+    if (cache_dtype == LI_F32) paged_store_kernel<float><<<T, 256, 0, stream>>>(src, stride, runs, slot_map, page_size);
+    else if (cache_dtype == LI_BF16) paged_store_kernel<bf16_t><<<T, 256, 0, stream>>>(src, stride, runs, slot_map, page_size);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// ------------------------------------------------------------------------------ difference of two attention maps
+// o = a1 - lambda * a2 per (token, head), then o / sqrt(mean(o^2) + eps) over the head's columns, times `mult`.
+// A wave a (token, head).
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void diff_combine_kernel(const TI* __restrict__ a1, const TI* __restrict__ a2, float lambda,
+                                                           float eps, float mult, TO* __restrict__ out, long pairs, int dv) {
+    const long pr = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pr >= pairs) return;
+    const int lane = threadIdx.x & 63;
+    const TI* r1 = a1 + (size_t)pr * dv;
+    const TI* r2 = a2 + (size_t)pr * dv;
+    float ss = 0.f;
+    for (int j = lane; j < dv; j += 64) {
+        const float o = fmaf(-lambda, load_as_float(r2 + j), load_as_float(r1 + j));
+        ss = fmaf(o, o, ss);
+    }
+    ss = wave_sum(ss);
+    const float f = mult / sqrtf(ss / (float)dv + eps);
+    for (int j = lane; j < dv; j += 64) {
+        const float o = fmaf(-lambda, load_as_float(r2 + j), load_as_float(r1 + j));
+        store_from_float(out + (size_t)pr * dv + j, o * f);
+    }
+}
+
+extern "C" int li_diff_combine(const void* a1, const void* a2, int in_dtype, float lambda, float eps, float mult, void* out,
+                               int out_dtype, long pairs, int dv, hipStream_t stream) {
+    if (pairs <= 0 || dv <= 0) return LI_ERR_SIZE;
+    const unsigned grid = (unsigned)((pairs + 3) / 4);
+#define DC(TI, TO) diff_combine_kernel<TI, TO><<<grid, 256, 0, stream>>>((const TI*)a1, (const TI*)a2, lambda, eps, mult, (TO*)out, pairs, dv)
+    if (in_dtype == LI_F32 && out_dtype == LI_F32) DC(float, float);
+    else if (in_dtype == LI_F32 && out_dtype == LI_BF16) DC(float, bf16_t);
+    else if (in_dtype == LI_BF16 && out_dtype == LI_BF16) DC(bf16_t, bf16_t);
+    else if (in_dtype == LI_BF16 && out_dtype == LI_F32) DC(bf16_t, float);
+    else return LI_ERR_DTYPE;
+#undef DC
+    return li_launch_status();
+}

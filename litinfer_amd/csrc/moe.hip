@@ -1,0 +1,305 @@
+// Routed feed-forward: the router (logits, the `top` largest, softmax over the chosen ones, and a sigmoid gate
+// for a shared expert), the plan of a step (the (token, choice) pairs sorted by expert, cut into tiles of rows),
+// the products of every tile's rows with its expert's matrix, and the weighted sum back into the stream.
+// Nothing here returns to the host: the numbers of rows an expert gets stay on the device, and the launches are
+// sized by what a step can have at most.
+#include "common.h"
+
+#define MOE_TILE 32            // rows of one expert that a tile holds
+
+// ------------------------------------------------------------------------------------------------ router
+// One block a token.  logits[e] = b[e] + sum_k W[e, k] x[k] in float32 (a wave an expert, in turns); the `top`
+// largest (the lower index wins a tie), weights = softmax over the chosen logits.  gate[t] = sigmoid(wg . x).
+template <typename TX, typename TW>
+__global__ __launch_bounds__(256) void moe_route_kernel(const TX* __restrict__ x, long x_stride, const TW* __restrict__ wr,
+                                                        const float* __restrict__ br, const TW* __restrict__ wg,
+                                                        int* __restrict__ idx, float* __restrict__ wt, float* __restrict__ gate,
+                                                        int K, int E, int top) {
+    extern __shared__ float sm[];                      // [K] the row, [E] the logits
+    float* xs = sm;
+    float* lg = sm + K;
+    const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const TX* row = x + (size_t)t * x_stride;
+    for (int k = threadIdx.x; k < K; k += 256) xs[k] = load_as_float(row + k);
+    __syncthreads();
+    for (int e = w; e < E + (wg ? 1 : 0); e += 4) {
+        const TW* wrow = e < E ? wr + (size_t)e * K : wg;
+        float s = 0.f;
+        for (int k = lane; k < K; k += 64) s = fmaf(load_as_float(wrow + k), xs[k], s);
+        s = wave_sum(s);
+        if (lane == 0) {
+            if (e < E) lg[e] = s + (br ? br[e] : 0.f);
+            else gate[t] = 1.0f / (1.0f + expf(-s));
+        }
+    }
+    __syncthreads();
+    if (w != 0) return;
+    // wave 0 picks: `top` rounds of a maximum over the logits that are left
+    float chosen = 0.f, mx = 0.f, sum = 0.f;
+    int mine = -1;
+    for (int r = 0; r < top; ++r) {
+        float best = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64) {
+            const float v = lg[e];
+            if (v > best || bi == 0x7fffffff) { best = v; bi = e; }            // (ascending e a lane: the first of equals stays)
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, LI_WAVE);
+            const int oi = __shfl_xor(bi, o, LI_WAVE);
+            if (oi != 0x7fffffff && (bi == 0x7fffffff || ob > best || (ob == best && oi < bi))) { best = ob; bi = oi; }
+        }
+        if (r == 0) mx = best;
+        const float ex = expf(best - mx);
+        sum += ex;
+        if (lane == r) { mine = bi; chosen = ex; }
+        if (lane == 0) lg[bi] = -INFINITY;
+        // (a wave's LDS instructions are carried out in the order of their issue: the next round reads what lane 0 wrote)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if (lane < top) { idx[(size_t)t * top + lane] = mine; wt[(size_t)t * top + lane] = chosen / sum; }
+}
+
+extern "C" int li_moe_route(const void* x, int x_dtype, long x_stride, const void* wr, int w_dtype, const float* br, const void* wg,
+                            int* idx, float* wt, float* gate, int T, int K, int E, int top, hipStream_t stream) {
+    if (T <= 0 || K <= 0 || E <= 0 || top <= 0 || top > E || top > 64 || x_stride < K || (size_t)(K + E) * 4 > 60000 || (wg && !gate))
+        return LI_ERR_SIZE;
+    const size_t lds = (size_t)(K + E) * 4;
+#define MR(TX, TW) moe_route_kernel<TX, TW><<<T, 256, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top)
+    if (x_dtype == LI_F32 && w_dtype == LI_F32) MR(float, float);
+    else if (x_dtype == LI_BF16 && w_dtype == LI_BF16) MR(bf16_t, bf16_t);
+    else if (x_dtype == LI_BF16 && w_dtype == LI_F32) MR(bf16_t, float);
+    else if (x_dtype == LI_F32 && w_dtype == LI_BF16) MR(float, bf16_t);
+    else return LI_ERR_DTYPE;
+#undef MR
+    return li_launch_status();
+}
+
+// -------------------------------------------------------------------------------------------------- plan
+// One block.  counts per expert, their running sum, every pair's row among its expert's rows (rows of an expert lie
+// together), and the tiles: (expert, first row, rows).  plan = [n_tiles, 0, 0, 0 | tiles x 4 | ...]; row_token[row] is
+// the token of a sorted row, pair_row[pair] the row of pair = token * top + choice.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ idx, int pairs, int top, int E, int* __restrict__ plan,
+                                                        int max_tiles, int* __restrict__ row_token, int* __restrict__ pair_row) {
+    extern __shared__ int si[];                         // [E] counts, then cursors; [E + 1] starts
+    int* cnt = si;
+    int* start = si + E;
+    for (int e = threadIdx.x; e < E; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < pairs; i += 1024) {
+        const int e = idx[i];
+        if (e >= 0 && e < E) atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, nt = 0;
+        for (int e = 0; e < E; ++e) {
+            start[e] = at;
+            for (int r = 0; r < cnt[e] && nt < max_tiles; r += MOE_TILE, ++nt) {
+                int* tile = plan + 4 + 4 * nt;
+                tile[0] = e; tile[1] = at + r; tile[2] = (cnt[e] - r < MOE_TILE) ? cnt[e] - r : MOE_TILE; tile[3] = 0;
+            }
+            at += cnt[e];
+        }
+        start[E] = at;
+        plan[0] = nt; plan[1] = at; plan[2] = plan[3] = 0;
+    }
+    __syncthreads();
+    // a pair's row: the next free one of its expert.  Which pair of an expert gets which of its rows depends on who
+    // comes first; a row's result does not depend on where it lies
+    for (int e = threadIdx.x; e < E; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < pairs; i += 1024) {
+        const int e = idx[i];
+        if (e >= 0 && e < E) {
+            const int row = start[e] + atomicAdd(&cnt[e], 1);
+            pair_row[i] = row;
+            row_token[row] = i / top;
+        } else {
+            pair_row[i] = -1;
+        }
+    }
+}
+
+extern "C" int li_moe_plan(const int* idx, int T, int top, int E, int* plan, int max_tiles, int* row_token, int* pair_row,
+                           hipStream_t stream) {
+    if (T <= 0 || top <= 0 || E <= 0 || E > 8000 || max_tiles <= 0) return LI_ERR_SIZE;
+    moe_plan_kernel<<<1, 1024, (size_t)(2 * E + 1) * 4, stream>>>(idx, T * top, top, E, plan, max_tiles, row_token, pair_row);
+    return li_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------- products by tile
+// out[row, j] = act(sum_k W[e, j, k] * a[src(row), k]) for the rows of every tile, e the tile's expert; src(row) =
+// row_token[row] where the rows are gathered from tokens, else the row itself.  act: 0 none, 1 max(., 0)^2.
+// General form: a block takes a tile and 64 outputs; rows and matrix rows go through LDS in float32, K in steps
+// of 32; a thread owns 2 rows x 4 outputs.  Sums are float32 in the order of k.
+template <typename TA, typename TW, typename TO>
+__global__ __launch_bounds__(256) void moe_linear_kernel(const TA* __restrict__ a, long a_stride, const int* __restrict__ row_token,
+                                                         const TW* __restrict__ w, const int* __restrict__ plan,
+                                                         TO* __restrict__ out, long out_stride, int n_out, int K, int act) {
+    const int tile = blockIdx.x;
+    if (tile >= plan[0]) return;
+    const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
+    const int j0 = blockIdx.y * 64;
+    __shared__ float As[MOE_TILE][33];
+    __shared__ float Ws[64][33];
+    __shared__ int src[MOE_TILE];
+    if (threadIdx.x < MOE_TILE) {
+        const int r = r0 + (threadIdx.x < nr ? threadIdx.x : 0);
+        src[threadIdx.x] = row_token ? row_token[r] : r;
+    }
+    const int tr = threadIdx.x / 16, tc = threadIdx.x % 16;          // rows 2 tr, 2 tr + 1; outputs tc + 16 i
+    float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    const TW* we = w + (size_t)e * n_out * K;
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < MOE_TILE * 32; i += 256) {
+            const int r = i / 32, k = k0 + i % 32;
+            As[r][i % 32] = (r < nr && k < K) ? load_as_float(a + (size_t)src[r] * a_stride + k) : 0.f;
+        }
+        for (int i = threadIdx.x; i < 64 * 32; i += 256) {
+            const int j = j0 + i / 32, k = k0 + i % 32;
+            Ws[i / 32][i % 32] = (j < n_out && k < K) ? load_as_float(we + (size_t)j * K + k) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int k = 0; k < 32; ++k) {
+            const float a0 = As[2 * tr][k], a1 = As[2 * tr + 1][k];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float wv = Ws[tc + 16 * i][k];
+                acc[0][i] = fmaf(a0, wv, acc[0][i]);
+                acc[1][i] = fmaf(a1, wv, acc[1][i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr) {
+        const int r = 2 * tr + rr;
+        if (r >= nr) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int j = j0 + tc + 16 * i;
+            if (j >= n_out) continue;
+            float v = acc[rr][i];
+            if (act == 1) { v = fmaxf(v, 0.f); v = v * v; }
+            store_from_float(out + (size_t)(r0 + r) * out_stride + j, v);
+        }
+    }
+}
+
+// The same on the matrix cores, for bfloat16 matrices with K a multiple of 16 and n_out a multiple of 32: a wave takes
+// the tile's 32 rows and 32 outputs and works on the transposed tile (outputs x rows), so that both operands are
+// 16-byte pieces of rows as they lie in memory and a lane ends with four consecutive outputs of its row.
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_f32x16 __attribute__((ext_vector_type(16)));
+union moe_frag8 { uint4 raw; uint32_t w[4]; moe_bf16x8 v; };
+
+template <typename TA, typename TO>
+__global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const TA* __restrict__ a, long a_stride, const int* __restrict__ row_token,
+                                                              const bf16_t* __restrict__ w, const int* __restrict__ plan,
+                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act) {
+    const int tile = blockIdx.x;
+    if (tile >= plan[0]) return;
+    const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ql = lane & 31, h2 = lane >> 5;
+    const int j0 = (blockIdx.y * 4 + wv) * 32;
+    if (j0 >= n_out) return;
+    const int r = r0 + (ql < nr ? ql : 0);
+    const int srow = row_token ? row_token[r] : r;
+    const TA* arow = a + (size_t)srow * a_stride + 8 * h2;
+    const bf16_t* mrow = w + ((size_t)e * n_out + j0 + ql) * K + 8 * h2;
+    moe_f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    for (int k = 0; k < K; k += 16) {
+        moe_frag8 fa, fb;
+        fa.raw = *reinterpret_cast<const uint4*>(mrow + k);
+        if constexpr (sizeof(TA) == 2) {
+            fb.raw = *reinterpret_cast<const uint4*>(arow + k);
+        } else {
+            const float4 u = *reinterpret_cast<const float4*>(arow + k);
+            const float4 v = *reinterpret_cast<const float4*>(arow + k + 4);
+            fb.w[0] = pack2_bf16(u.x, u.y); fb.w[1] = pack2_bf16(u.z, u.w);
+            fb.w[2] = pack2_bf16(v.x, v.y); fb.w[3] = pack2_bf16(v.z, v.w);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, fb.v, acc, 0, 0, 0);
+    }
+    if (ql >= nr) return;
+    TO* orow = out + (size_t)(r0 + ql) * out_stride + j0;
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {                   // registers 4 rg .. 4 rg + 3: outputs 8 rg + 4 h2 ..
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = acc[4 * rg + i];
+            if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
+        }
+        TO* dst = orow + 8 * rg + 4 * h2;
+        if constexpr (sizeof(TO) == 2) {
+            uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
+            d2[0] = pack2_bf16(v[0], v[1]);
+            d2[1] = pack2_bf16(v[2], v[3]);
+        } else {
+            *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+        }
+    }
+}
+
+extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const int* row_token, const void* w, int w_dtype,
+                             const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act,
+                             hipStream_t stream) {
+    if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || out_stride < n_out || act < 0 || act > 1) return LI_ERR_SIZE;
+    if (w_dtype == LI_BF16 && K % 16 == 0 && n_out % 32 == 0 && a_stride % 8 == 0 && out_stride % 4 == 0 &&
+        ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0 && (a_dtype == LI_BF16 || a_dtype == LI_F32)) {
+        const dim3 grid(max_tiles, (n_out + 127) / 128);
+#define MM(TA, TO) moe_linear_mfma_kernel<TA, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act)
+        if (a_dtype == LI_BF16 && out_dtype == LI_BF16) MM(bf16_t, bf16_t);
+        else if (a_dtype == LI_BF16 && out_dtype == LI_F32) MM(bf16_t, float);
+        else if (a_dtype == LI_F32 && out_dtype == LI_BF16) MM(float, bf16_t);
+        else if (a_dtype == LI_F32 && out_dtype == LI_F32) MM(float, float);
+        else return LI_ERR_DTYPE;
+#undef MM
+        return li_launch_status();
+    }
+    const dim3 grid(max_tiles, (n_out + 63) / 64);
+#define ML(TA, TW, TO) moe_linear_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const TW*)w, plan, (TO*)out, out_stride, n_out, K, act)
+    if (a_dtype == LI_F32 && w_dtype == LI_F32 && out_dtype == LI_F32) ML(float, float, float);
+    else if (a_dtype == LI_BF16 && w_dtype == LI_BF16 && out_dtype == LI_BF16) ML(bf16_t, bf16_t, bf16_t);
+    else if (a_dtype == LI_BF16 && w_dtype == LI_BF16 && out_dtype == LI_F32) ML(bf16_t, bf16_t, float);
+    else if (a_dtype == LI_F32 && w_dtype == LI_BF16 && out_dtype == LI_F32) ML(float, bf16_t, float);
+    else if (a_dtype == LI_F32 && w_dtype == LI_BF16 && out_dtype == LI_BF16) ML(float, bf16_t, bf16_t);
+    else return LI_ERR_DTYPE;
+#undef ML
+    return li_launch_status();
+}
+
+// ----------------------------------------------------------------------------------------------- the sum
+// x[t, :] += sum_c wt[t, c] * yrow[pair_row[t * top + c], :] (in the order of c) + gate[t] * shared[t, :].
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, long x_stride, const float* __restrict__ yrows,
+                                                          long y_stride, const int* __restrict__ pair_row, const float* __restrict__ wt,
+                                                          const float* __restrict__ gate, const float* __restrict__ shared_out,
+                                                          long s_stride, int H, int top) {
+    const int t = blockIdx.x;
+    for (int j = blockIdx.y * 256 + threadIdx.x; j < H; j += gridDim.y * 256) {
+        float s = 0.f;
+        for (int c = 0; c < top; ++c) {
+            const int row = pair_row[(size_t)t * top + c];
+            if (row >= 0) s = fmaf(wt[(size_t)t * top + c], yrows[(size_t)row * y_stride + j], s);
+        }
+        if (shared_out) s = fmaf(gate ? gate[t] : 1.f, shared_out[(size_t)t * s_stride + j], s);
+        x[(size_t)t * x_stride + j] += s;
+    }
+}
+
+extern "C" int li_moe_combine(float* x, long x_stride, const float* yrows, long y_stride, const int* pair_row, const float* wt,
+                              const float* gate, const float* shared_out, long s_stride, int T, int H, int top, hipStream_t stream) {
+    if (T <= 0 || H <= 0 || top <= 0 || x_stride < H || y_stride < H || (shared_out && s_stride < H)) return LI_ERR_SIZE;
+    int ys = (H + 255) / 256;
+    if (ys > 64) ys = 64;
+    moe_combine_kernel<<<dim3(T, ys), 256, 0, stream>>>(x, x_stride, yrows, y_stride, pair_row, wt, gate, shared_out, s_stride, H, top);
+    return li_launch_status();
+}

@@ -1,0 +1,381 @@
+// Kernels of recurrent mixers whose state has a fixed size per request: a short causal convolution
+// per channel with its tail of past inputs, the selective state-space recurrence
+//   S_t = a_t S_{t-1} + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t,  a_t = exp(-exp(A_log) dt_t),
+// and the gated RMS norm in groups of columns behind it.  Everything here is float32: inputs, decays,
+// step sizes, the state and the sums; only the normed output is rounded to the activations' type.
+#include "common.h"
+
+// ------------------------------------------------------------------------------------ causal convolution
+// out[t, c] = silu(b[c] + sum_j w[c, j] * u[t - (taps - 1 - j), c]): the last column of w multiplies the
+// current token.  Inputs before the first token of the step's portion come from the request's tail
+// [slots, taps - 1, C] (its last taps - 1 inputs, zeros for a new request).
+__global__ __launch_bounds__(256) void causal_conv_silu_kernel(
+    const float* __restrict__ u, long u_stride, int C, int taps, const float* __restrict__ w, const float* __restrict__ b,
+    const float* __restrict__ tail, const int* __restrict__ seg_of_token, const int* __restrict__ q_start,
+    const int* __restrict__ slots, float* __restrict__ out, long out_stride) {
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int seg = seg_of_token[t], i = t - q_start[seg], slot = slots[seg];
+    float acc = b ? b[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j, li = i - back;
+        const float v = li >= 0 ? u[(size_t)(t - back) * u_stride + c]
+                                : tail[((size_t)slot * (taps - 1) + (taps - 1 + li)) * C + c];
+        acc = fmaf(w[(size_t)c * taps + j], v, acc);
+    }
+    out[(size_t)t * out_stride + c] = acc / (1.0f + expf(-acc));
+}
+
+// The tail after the step: the last taps - 1 inputs of the request, those of this portion and, where it is
+// shorter than that, what is left of the old tail.  A thread owns a (request, channel) and goes upwards, so
+// it never reads what it has written.
+__global__ __launch_bounds__(256) void conv_tail_update_kernel(
+    const float* __restrict__ u, long u_stride, int C, int taps, float* __restrict__ tail,
+    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ slots) {
+    const int seg = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int L = q_len[seg], t0 = q_start[seg];
+    float* mine = tail + (size_t)slots[seg] * (taps - 1) * C + c;
+    for (int r = 0; r < taps - 1; ++r) {
+        const int li = L - (taps - 1) + r;
+        mine[(size_t)r * C] = li >= 0 ? u[(size_t)(t0 + li) * u_stride + c] : mine[(size_t)(r + L) * C];
+    }
+}
+
+extern "C" int li_causal_conv_silu(const float* u, long u_stride, int C, int taps, const float* w, const float* b, float* tail,
+                                   const int* seg_of_token, const int* q_start, const int* q_len, const int* slots,
+                                   float* out, long out_stride, int T, int segs, hipStream_t stream) {
+    if (T <= 0 || segs <= 0 || C <= 0 || taps <= 0 || taps > 64 || u_stride < C || out_stride < C) return LI_ERR_SIZE;
+    const dim3 grid(T, (C + 255) / 256);
+    causal_conv_silu_kernel<<<grid, 256, 0, stream>>>(u, u_stride, C, taps, w, b, tail, seg_of_token, q_start, slots, out, out_stride);
+    if (taps > 1) {
+        const dim3 g2(segs, (C + 255) / 256);
+        conv_tail_update_kernel<<<g2, 256, 0, stream>>>(u, u_stride, C, taps, tail, q_start, q_len, slots);
+    }
+    return li_launch_status();
+}
+
+// ------------------------------------------------------------------------------------ state-space recurrence
+// A column p of a head's state (its N values) evolves by itself, given x_t[p] and the head's a_t, dt_t, B_t,
+// C_t.  A lane owns NR state values of one column in registers: lane = column * NS + slice, the slices of a
+// column are NS neighbouring lanes that add their shares of y up.  A wave is 64 / NS columns of one head; the
+// four waves of a block are heads (or column ranges) of ONE group and share its B_t and C_t, which lie in LDS
+// for SSM_TB tokens at a time beside each wave's x_t, dt_t and a_t.
+//
+// A step's portion of a request is cut into chunks of Q tokens that run side by side:
+//   MODE 1: the state that a chunk alone builds up from zero, and the product of its decays;
+//   the carry kernel: the state with which every chunk begins, chunk after chunk;
+//   MODE 0: the recurrence itself from that state, with the outputs; the last chunk leaves the request's state.
+// A portion of at most Q tokens (a decoding step) is MODE 0 alone, from the request's state.
+#define SSM_TB 16
+#define SSM_WAVES 4
+
+__device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+template <int NR, int NS, int MODE>
+__global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_kernel(
+    const float* __restrict__ xbc, long xbc_stride, const float* __restrict__ dt_raw, long dt_stride,
+    const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dw,
+    float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ q_start, const int* __restrict__ q_len,
+    const int* __restrict__ chunk_seg, const int* __restrict__ chunk_idx, float* __restrict__ carry, float* __restrict__ decay,
+    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, int Q) {
+    constexpr int NP = NR * NS, PW = 64 / NS;
+    extern __shared__ __align__(16) float lds[];
+    float* sB = lds;                                   // [SSM_TB][NP]
+    float* sC = sB + SSM_TB * NP;                      // [SSM_TB][NP]
+    float* sX = sC + SSM_TB * NP;                      // [SSM_WAVES][SSM_TB][PW]
+    float* sDt = sX + SSM_WAVES * SSM_TB * PW;         // [SSM_WAVES][SSM_TB]
+    float* sA = sDt + SSM_WAVES * SSM_TB;              // [SSM_WAVES][SSM_TB]
+    const int bx = blockIdx.x;
+    const int seg = chunk_seg ? chunk_seg[bx] : bx;
+    if (seg < 0) return;
+    const int c = chunk_seg ? chunk_idx[bx] : 0;
+    const int L = q_len[seg], first = c * Q;
+    if (first >= L) return;
+    const int ntok = (L - first < Q) ? L - first : Q;
+    const bool last = first + ntok >= L;
+    if (MODE == 1 && last) return;                      // nobody needs the last chunk's own state
+    const int t0 = q_start[seg] + first;
+    const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
+    const int g = blockIdx.y / ublocks, ub = blockIdx.y % ublocks;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int unit = ub * SSM_WAVES + w;
+    const bool active = unit < U;
+    const int head = g * hpg + (active ? unit / PS : 0), pbase = active ? (unit % PS) * PW : 0;
+    const int pl = lane / NS, s = lane % NS, p = pbase + pl;
+    const int inner = heads * vdim;
+    const size_t hoff = (size_t)head * N * vdim;
+    float S[NR];
+    if (MODE == 0 && active) {
+        const float* src = chunk_seg ? carry + (size_t)bx * heads * N * vdim + hoff
+                                     : state + (size_t)slots[seg] * heads * N * vdim + hoff;
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int n = s * NR + r;
+            S[r] = (n < N && p < vdim) ? src[(size_t)n * vdim + p] : 0.f;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) S[r] = 0.f;
+    }
+    float prod = 1.f;
+    const float Dh = (MODE == 0 && active) ? Dw[head] : 0.f;
+    for (int b0 = 0; b0 < ntok; b0 += SSM_TB) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < SSM_TB * NP; i += 64 * SSM_WAVES) {
+            const int tt = i / NP, n = i % NP;
+            const bool ok = b0 + tt < ntok && n < N;
+            const float* row = xbc + (size_t)(t0 + b0 + tt) * xbc_stride + inner + (size_t)g * N + n;
+            sB[i] = ok ? row[0] : 0.f;
+            sC[i] = ok ? row[(size_t)G * N] : 0.f;
+        }
+        if (active) {
+            for (int i = lane; i < SSM_TB * PW; i += 64) {
+                const int tt = i / PW, pp = pbase + i % PW;
+                const bool ok = b0 + tt < ntok && pp < vdim;
+                sX[(w * SSM_TB + tt) * PW + i % PW] = ok ? xbc[(size_t)(t0 + b0 + tt) * xbc_stride + (size_t)head * vdim + pp] : 0.f;
+            }
+            if (lane < SSM_TB) {
+                const bool ok = b0 + lane < ntok;
+                const float d = ok ? softplus_f32(dt_raw[(size_t)(t0 + b0 + lane) * dt_stride + head] + dt_bias[head]) : 0.f;
+                sDt[w * SSM_TB + lane] = d;
+                sA[w * SSM_TB + lane] = expf(-expf(A_log[head]) * d);
+            }
+        }
+        __syncthreads();
+        if (!active) continue;
+        const int nt = (ntok - b0 < SSM_TB) ? ntok - b0 : SSM_TB;
+        for (int tt = 0; tt < nt; ++tt) {
+            const float a = sA[w * SSM_TB + tt], dtv = sDt[w * SSM_TB + tt];
+            const float xv = sX[(w * SSM_TB + tt) * PW + pl];
+            const float dx = dtv * xv;
+            const float4* Bp = reinterpret_cast<const float4*>(sB + tt * NP + s * NR);
+            const float4* Cp = reinterpret_cast<const float4*>(sC + tt * NP + s * NR);
+            float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
+#pragma unroll
+            for (int r4 = 0; r4 < NR / 4; ++r4) {
+                const float4 bv = Bp[r4];
+                S[4 * r4 + 0] = fmaf(a, S[4 * r4 + 0], bv.x * dx);
+                S[4 * r4 + 1] = fmaf(a, S[4 * r4 + 1], bv.y * dx);
+                S[4 * r4 + 2] = fmaf(a, S[4 * r4 + 2], bv.z * dx);
+                S[4 * r4 + 3] = fmaf(a, S[4 * r4 + 3], bv.w * dx);
+                if (MODE == 0) {
+                    const float4 cv = Cp[r4];
+                    y0 = fmaf(S[4 * r4 + 0], cv.x, y0);
+                    y1 = fmaf(S[4 * r4 + 1], cv.y, y1);
+                    y2 = fmaf(S[4 * r4 + 2], cv.z, y2);
+                    y3 = fmaf(S[4 * r4 + 3], cv.w, y3);
+                }
+            }
+            if (MODE == 0) {
+                float yv = (y0 + y1) + (y2 + y3);
+#pragma unroll
+                for (int o = 1; o < NS; o <<= 1) yv += __shfl_xor(yv, o, LI_WAVE);
+                if (s == 0 && p < vdim) y[(size_t)(t0 + b0 + tt) * y_stride + (size_t)head * vdim + p] = fmaf(Dh, xv, yv);
+            } else {
+                prod *= a;
+            }
+        }
+    }
+    if (!active) return;
+    float* dst = nullptr;
+    if (MODE == 1) {
+        dst = carry + (size_t)bx * heads * N * vdim + hoff;
+        if (lane == 0 && pbase == 0) decay[(size_t)bx * heads + head] = prod;
+    } else if (last) {
+        dst = state + (size_t)slots[seg] * heads * N * vdim + hoff;
+    }
+    if (dst) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int n = s * NR + r;
+            if (n < N && p < vdim) dst[(size_t)n * vdim + p] = S[r];
+        }
+    }
+}
+
+// Numbers the chunks of a step: request after request, chunk after chunk.  chunk_first[seg] is a request's
+// first chunk; chunk_seg / chunk_idx say whose chunk, and which of its chunks, a number is (-1: none).
+__global__ __launch_bounds__(256) void ssm_chunk_index_kernel(const int* __restrict__ q_len, int segs, int Q, int max_chunks,
+                                                              int* __restrict__ chunk_seg, int* __restrict__ chunk_idx,
+                                                              int* __restrict__ chunk_first) {
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int sgm = 0; sgm < segs; ++sgm) {
+            chunk_first[sgm] = at;
+            at += (q_len[sgm] + Q - 1) / Q;
+        }
+        chunk_first[segs] = at;
+    }
+    for (int i = threadIdx.x; i < max_chunks; i += 256) chunk_seg[i] = -1;
+    __syncthreads();
+    for (int sgm = threadIdx.x; sgm < segs; sgm += 256) {
+        const int f = chunk_first[sgm], n = chunk_first[sgm + 1] - f;
+        for (int k = 0; k < n && f + k < max_chunks; ++k) { chunk_seg[f + k] = sgm; chunk_idx[f + k] = k; }
+    }
+}
+
+// carry[chunk] holds what the chunk alone built up from zero; afterwards it holds the state with which the
+// chunk begins: the request's state for its first chunk, decay * (state before) + (built up before) onwards.
+__global__ __launch_bounds__(256) void ssm_carry_kernel(float* __restrict__ carry, const float* __restrict__ decay,
+                                                        const float* __restrict__ state, const int* __restrict__ slots,
+                                                        const int* __restrict__ q_len, const int* __restrict__ chunk_first,
+                                                        int heads, int NV, int Q) {
+    const int seg = blockIdx.x, head = blockIdx.y;
+    const int nch = (q_len[seg] + Q - 1) / Q, base = chunk_first[seg];
+    const float* st = state + ((size_t)slots[seg] * heads + head) * NV;
+    for (int e = blockIdx.z * 256 + threadIdx.x; e < NV; e += gridDim.z * 256) {
+        float run = st[e];
+        for (int k = 0; k < nch; ++k) {
+            float* at = carry + ((size_t)(base + k) * heads + head) * NV + e;
+            float next = 0.f;
+            if (k + 1 < nch) next = fmaf(decay[(size_t)(base + k) * heads + head], run, *at);
+            *at = run;
+            run = next;
+        }
+    }
+}
+
+template <int NR, int NS>
+static int ssm_launch(const float* xbc, long xbc_stride, const float* dt_raw, long dt_stride, const float* dt_bias,
+                      const float* A_log, const float* Dw, float* state, const int* slots, const int* q_start, const int* q_len,
+                      int* chunk_tab, float* carry, float* decay, float* y, long y_stride, int heads, int vdim, int N, int G,
+                      int Q, int segs, int max_chunks, bool chunked, hipStream_t stream) {
+    constexpr int NP = NR * NS, PW = 64 / NS;
+    const size_t lds = (size_t)(2 * SSM_TB * NP + SSM_WAVES * SSM_TB * PW + 2 * SSM_WAVES * SSM_TB) * sizeof(float);
+    const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
+    if (!chunked) {
+        const dim3 grid(segs, G * ublocks);
+        ssm_scan_kernel<NR, NS, 0><<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
+            state, slots, q_start, q_len, nullptr, nullptr, nullptr, nullptr, y, y_stride, heads, vdim, N, G, Q);
+        return li_launch_status();
+    }
+    int* chunk_seg = chunk_tab;
+    int* chunk_idx = chunk_tab + max_chunks;
+    int* chunk_first = chunk_tab + 2 * max_chunks;
+    ssm_chunk_index_kernel<<<1, 256, 0, stream>>>(q_len, segs, Q, max_chunks, chunk_seg, chunk_idx, chunk_first);
+    const dim3 grid(max_chunks, G * ublocks);
+    ssm_scan_kernel<NR, NS, 1><<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
+        state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q);
+    const int NV = N * vdim;
+    int zs = (NV + 255) / 256;
+    if (zs > 16) zs = 16;
+    ssm_carry_kernel<<<dim3(segs, heads, zs), 256, 0, stream>>>(carry, decay, state, slots, q_len, chunk_first, heads, NV, Q);
+    ssm_scan_kernel<NR, NS, 0><<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
+        state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q);
+    return li_launch_status();
+}
+
+// How a state of N values a column is spread: slices (lanes a column) and values a lane; 0 if no kernel has it.
+extern "C" int li_ssm_scan_layout(int N, int vdim, int* slices, int* per_lane) {
+    if (N <= 0 || N > 256 || vdim <= 0) return 0;
+    int ns = 1;
+    while (ns < 4 && 64 / (2 * ns) >= vdim) ns *= 2;        // few columns a head: more lanes a column, so that a wave is full
+    while (ns < 4 && (N + ns - 1) / ns > 128) ns *= 2;
+    const int need = (N + ns - 1) / ns;
+    int nr = need <= 16 ? 16 : need <= 32 ? 32 : need <= 64 ? 64 : need <= 128 ? 128 : 0;
+    if (!nr) return 0;
+    while (ns * nr > 256 && ns > 1 && (N + ns / 2 - 1) / (ns / 2) <= 128) {     // no more padding than LDS has room for
+        ns /= 2;
+        const int nd = (N + ns - 1) / ns;
+        nr = nd <= 16 ? 16 : nd <= 32 ? 32 : nd <= 64 ? 64 : 128;
+    }
+    if (ns * nr > 256) return 0;
+    if (slices) *slices = ns;
+    if (per_lane) *per_lane = nr;
+    return 1;
+}
+
+// Chunks that a step of T tokens in `segs` portions can have at most, and the bytes of the tables and states
+// that the chunked form keeps in the workspace.
+extern "C" long li_ssm_scan_work_bytes(int T, int segs, int heads, int vdim, int N, int Q, int* max_chunks) {
+    const long mc = (long)T / Q + segs;
+    if (max_chunks) *max_chunks = (int)mc;
+    const long ints = ((3 * mc + segs + 1 + 3) / 4) * 4;
+    return ints * 4 + mc * heads * ((long)N * vdim + 1) * 4;
+}
+
+extern "C" int li_ssm_scan(const float* xbc, long xbc_stride, const float* dt_raw, long dt_stride, const float* dt_bias,
+                           const float* A_log, const float* Dw, float* state, const int* slots, const int* q_start,
+                           const int* q_len, float* y, long y_stride, int heads, int vdim, int N, int G, int Q, int T,
+                           int segs, int max_q_len, void* work, long work_bytes, hipStream_t stream) {
+    if (T <= 0 || segs <= 0 || heads <= 0 || G <= 0 || heads % G || vdim <= 0 || N <= 0 || Q <= 0 || max_q_len <= 0 ||
+        xbc_stride < (long)heads * vdim + 2L * G * N || dt_stride < heads || y_stride < (long)heads * vdim)
+        return LI_ERR_SIZE;
+    int ns = 0, nr = 0;
+    if (!li_ssm_scan_layout(N, vdim, &ns, &nr)) return LI_ERR_SIZE;
+    const bool chunked = max_q_len > Q;
+    int max_chunks = 0;
+    int* chunk_tab = nullptr;
+    float *carry = nullptr, *decay = nullptr;
+    if (chunked) {
+        const long need = li_ssm_scan_work_bytes(T, segs, heads, vdim, N, Q, &max_chunks);
+        if (!work || work_bytes < need || ((uintptr_t)work % 16)) return LI_ERR_SIZE;
+        chunk_tab = (int*)work;
+        const long ints = ((3L * max_chunks + segs + 1 + 3) / 4) * 4;
+        carry = (float*)work + ints;
+        decay = carry + (size_t)max_chunks * heads * N * vdim;
+    }
+#define SSM_GO(NR_, NS_)                                                                                                  \
+    if (nr == NR_ && ns == NS_)                                                                                           \
+        return ssm_launch<NR_, NS_>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw, state, slots, q_start, q_len,    \
+                                    chunk_tab, carry, decay, y, y_stride, heads, vdim, N, G, Q, segs, max_chunks, chunked, stream);
+    SSM_GO(16, 1) SSM_GO(32, 1) SSM_GO(64, 1) SSM_GO(128, 1)
+    SSM_GO(16, 2) SSM_GO(32, 2) SSM_GO(64, 2) SSM_GO(128, 2)
+    SSM_GO(16, 4) SSM_GO(32, 4) SSM_GO(64, 4)
+#undef SSM_GO
+    return LI_ERR_SIZE;
+}
+
+// ------------------------------------------------------------------------------------ gated norm in groups
+// out[t, c] = w[c] * v / sqrt(mean over c's group of v^2 + eps), v = y[t, c] * silu(z[t, c]): the gate comes
+// before the norm; every group of `gs` neighbouring columns has its own root mean square.  A block a (token, group).
+template <typename TO, int PER>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, long y_stride,
+                                                               const float* __restrict__ z, long z_stride,
+                                                               const float* __restrict__ w, float eps, TO* __restrict__ out,
+                                                               long out_stride, int gs) {
+    __shared__ float red[256 / LI_WAVE];
+    const int t = blockIdx.x, c0 = blockIdx.y * gs;
+    const float* yr = y + (size_t)t * y_stride + c0;
+    const float* zr = z + (size_t)t * z_stride + c0;
+    float v[PER];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * 256;
+        float g = 0.f;
+        if (j < gs) { const float zz = zr[j]; g = yr[j] * (zz / (1.0f + expf(-zz))); }
+        v[i] = g;
+        ss += g * g;
+    }
+    for (int j = threadIdx.x + PER * 256; j < gs; j += 256) {
+        const float zz = zr[j], g = yr[j] * (zz / (1.0f + expf(-zz)));
+        ss += g * g;
+    }
+    ss = block_sum<256>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+    TO* o = out + (size_t)t * out_stride + c0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * 256;
+        if (j < gs) store_from_float(o + j, w[c0 + j] * v[i] * inv);
+    }
+    for (int j = threadIdx.x + PER * 256; j < gs; j += 256) {
+        const float zz = zr[j], g = yr[j] * (zz / (1.0f + expf(-zz)));
+        store_from_float(o + j, w[c0 + j] * g * inv);
+    }
+}
+
+extern "C" int li_gated_group_norm(const float* y, long y_stride, const float* z, long z_stride, const float* w, float eps,
+                                   void* out, int out_dtype, long out_stride, int T, int n, int groups, hipStream_t stream) {
+    if (T <= 0 || n <= 0 || groups <= 0 || n % groups || groups > 65535 || y_stride < n || z_stride < n || out_stride < n)
+        return LI_ERR_SIZE;
+    const dim3 grid(T, groups);
+    if (out_dtype == LI_F32)
+        gated_group_norm_kernel<float, 8><<<grid, 256, 0, stream>>>(y, y_stride, z, z_stride, w, eps, (float*)out, out_stride, n / groups);
+    else if (out_dtype == LI_BF16)
+        gated_group_norm_kernel<bf16_t, 8><<<grid, 256, 0, stream>>>(y, y_stride, z, z_stride, w, eps, (bf16_t*)out, out_stride, n / groups);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
+}

@@ -77,6 +77,10 @@ class StepContext:
         self.feedback: torch.Tensor = None            # the engine's buffer of ids chosen on the device
         self.positions: torch.Tensor = None
         self.state_slots: torch.Tensor = None        # [segments] int32, device
+        self.seg_of_token: torch.Tensor = None       # [T] int32, device: the segment of every token
+        self.q_start: torch.Tensor = None            # [segments] int32, device: a segment's first token of the step
+        self.q_len: torch.Tensor = None              # [segments] int32, device: its tokens in this step
+        self.max_q_len = 0                           # the longest segment of the step (a host number: sizes launches)
         self.host_state_slots: np.ndarray = None
         self.host_q_start: np.ndarray = None
         self.host_q_len: np.ndarray = None
@@ -172,6 +176,7 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     ctx.ids, ctx.positions = d(0, T), d(1, T)
     d_seg, d_qs, d_ql, d_cl = d(2, T), d(3, nseg), d(4, nseg), d(5, nseg)
     ctx.state_slots, ctx.want_rows = d(6, nseg), d(7, nwant)
+    ctx.seg_of_token, ctx.q_start, ctx.q_len, ctx.max_q_len = d_seg, d_qs, d_ql, max_q
     d_single = d(8, nsingle) if token_kinds else None
     d_multi = d(9, nmulti) if token_kinds else None
     d_tiles = d(10, ntiles * 4, (ntiles, 4)) if tile_rows else None

@@ -383,7 +383,7 @@ class Engine:
         seen = 1 if state is None else state[1] + 1
         graphs[key] = ("seen", seen)
         graphs.move_to_end(key)
-        logits = None
+        logits, ran = None, False                 # (a step without wanted rows has no logits: `ran` says whether it has run)
         if seen >= self.graph_after:
             made = self.ws.allocations
             graph, out = self._record(ctx)
@@ -397,8 +397,8 @@ class Engine:
                 graphs[key] = ("graph", graph, out)
                 self.graphs_recorded += 1
                 graph.replay()
-                logits = out
-        if logits is None:
+                logits, ran = out, True
+        if not ran:
             logits = self.model.forward(ctx, self.cache)
             if self._graph_generation != self._buffers_at():
                 # this pass itself made a buffer grow (a larger batch than any before): what was

@@ -84,7 +84,7 @@ class Model:
         float32 logits [wanted, vocab] at the wanted rows (None if none)."""
         h = self.spec.hidden_size
         x = ctx.ws.buffer("model.residual", (ctx.num_tokens, h), torch.float32)
-        self.embedding.forward(ctx.ids, x, ctx.id_src, ctx.feedback)
+        self.embedding.forward(ctx.ids, x, ctx.id_src, ctx.feedback, positions=ctx.positions)
         stream = ResidualStream(x, ctx.ws)
         stream.ws_dtype = self.rt.dtype
         for i, e in enumerate(self.order):

@@ -36,7 +36,7 @@ MODULE_FLAGS = {"attention": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
                 # list, which the compiler remarks upon for every instance
                 "gemm": ["-Wno-inline-asm"]}
 
-MODULES = ("elementwise", "gemm", "attention", "attention_masked", "sampling", "host")     # what the models need
+MODULES = ("elementwise", "gemm", "attention", "attention_masked", "recurrent", "moe", "sampling", "host")     # what the models need
 # measuring kernels of the benchmark (a streaming read, a copy, a matrix-core loop): built with the
 # rest by `build_all(everything=True)`, otherwise when the benchmark first asks for them
 EXTRA_MODULES = ("probe",)

@@ -44,6 +44,21 @@ _SIGNATURES = {
         "li_rope_pairs_apply": [P, I, I, I, I, I, P, P, I],
         "li_qk_norm_pairs_store": [P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, I],
         "li_latent_norm_pairs_store": [P, I, I, I, I, I, P, F, P, P, P, P, I, P, I, I],
+        "li_sinusoid_add": [P, P, P, I, I],
+        "li_scale_softcap": [P, L, F, F],
+        "li_paged_store": [P, L, I, I, I, P, I, I, I, P, I, I, I, P, I, P, I, I],
+        "li_diff_combine": [P, P, I, F, F, F, P, I, L, I],
+    },
+    "recurrent": {
+        "li_causal_conv_silu": [P, L, I, I, P, P, P, P, P, P, P, P, L, I, I],
+        "li_ssm_scan": [P, L, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, P, L],
+        "li_gated_group_norm": [P, L, P, L, P, F, P, I, L, I, I, I],
+    },
+    "moe": {
+        "li_moe_route": [P, I, L, P, I, P, P, P, P, P, I, I, I, I],
+        "li_moe_plan": [P, I, I, I, P, I, P, P],
+        "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I],
+        "li_moe_combine": [P, L, P, L, P, P, P, P, L, I, I, I],
     },
     "attention_masked": {
         "li_masked_attention": [P, I, I, P, I, P, P, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, F, F, I],
@@ -1285,3 +1300,209 @@ def sample_prepare(rows: torch.Tensor, table: torch.Tensor, temperature: torch.T
     if n:
         _run("sampling", "li_sample_prepare", rows.data_ptr(), n, table.data_ptr(), table.shape[0],
              temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr())
+
+
+# ------------------------------------------------------------- position vector, logits, pages, map difference
+def sinusoid_add(x: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor) -> None:
+    """x[t, 2i] += sin(p f_i), x[t, 2i + 1] += cos(p f_i) for p = positions[t]; freq float32 [ceil(H / 2)]."""
+    _gpu(x, positions, freq)
+    t, h = x.shape
+    _chk(x.dtype is torch.float32 and x.is_contiguous() and positions.dtype is torch.int32 and positions.numel() == t
+         and positions.is_contiguous() and freq.dtype is torch.float32 and freq.is_contiguous()
+         and freq.numel() == (h + 1) // 2, "sinusoid_add: x [T, H] float32, positions [T] int32, freq [ceil(H / 2)] float32")
+    if t:
+        _run("elementwise", "li_sinusoid_add", x.data_ptr(), positions.data_ptr(), freq.data_ptr(), t, h)
+
+
+def scale_softcap(x: torch.Tensor, scale: float, cap: float) -> None:
+    """x <- x * scale, then cap * tanh(x / cap) where cap > 0; in place, float32."""
+    _gpu(x)
+    _chk(x.dtype is torch.float32 and x.is_contiguous() and cap >= 0, "scale_softcap: a contiguous float32 tensor, cap >= 0")
+    if x.numel():
+        _run("elementwise", "li_scale_softcap", x.data_ptr(), x.numel(), float(scale), float(cap))
+
+
+def paged_store(src: torch.Tensor, runs, slot_map: torch.Tensor, page_size: int) -> None:
+    """Up to three runs (first column, heads, columns a head, paged tensor [pages, heads, page_size, columns]) of the
+    float32 rows `src` [T, stride] go to every token's slot."""
+    t = src.shape[0]
+    _gpu(src, slot_map, *(r[3] for r in runs))
+    _chk(src.dtype is torch.float32 and _rows_ok(src) and slot_map.dtype is torch.int32 and slot_map.numel() == t
+         and slot_map.is_contiguous() and 1 <= len(runs) <= 3, "paged_store: src [T, stride] float32, slot_map [T] int32, 1 to 3 runs")
+    dt = runs[0][3].dtype
+    flat = []
+    for col, heads, dim, dst in runs:
+        _chk(dst.dtype is dt and dt in _DT and dst.dim() == 4 and dst.is_contiguous() and dst.shape[1:] == (heads, page_size, dim)
+             and 0 <= col and col + heads * dim <= src.shape[1], "paged_store: a run does not fit its rows or its pages")
+        flat += [int(col), int(heads), int(dim), dst.data_ptr()]
+    flat += [0, 0, 0, 0] * (3 - len(runs))
+    if t:
+        _run("elementwise", "li_paged_store", src.data_ptr(), src.stride(0), *flat, _DT[dt], slot_map.data_ptr(), int(page_size), t)
+
+
+def diff_combine(a1: torch.Tensor, a2: torch.Tensor, lam: float, eps: float, mult: float, out: torch.Tensor, dv: int) -> None:
+    """out = mult * o / sqrt(mean(o^2) + eps) over every head's dv columns, o = a1 - lam * a2; all [T, heads * dv]."""
+    _gpu(a1, a2, out)
+    _chk(a1.shape == a2.shape == out.shape and a1.dtype is a2.dtype and a1.dtype in _DT and out.dtype in _DT
+         and a1.is_contiguous() and a2.is_contiguous() and out.is_contiguous() and dv > 0 and a1.shape[1] % dv == 0,
+         "diff_combine: a1, a2, out [T, heads * dv]")
+    if a1.numel():
+        _run("elementwise", "li_diff_combine", a1.data_ptr(), a2.data_ptr(), _DT[a1.dtype], float(lam), float(eps), float(mult),
+             out.data_ptr(), _DT[out.dtype], a1.numel() // dv, int(dv))
+
+
+# ------------------------------------------------------------------------------------------ recurrent mixers
+SSM_CHUNK = 64          # tokens of a portion that one block of the recurrence takes; longer portions run as chunks side by side
+
+
+def _lib_fn(module: str, name: str, argtypes, restype):
+    f = _fn_cache.get((module, name))
+    if f is None:
+        f = getattr(build.load(module), name)
+        f.argtypes, f.restype = argtypes, restype
+        _fn_cache[(module, name)] = f
+    return f
+
+
+def ssm_scan_takes(state: int, vdim: int) -> bool:
+    """Whether the recurrence kernel has a layout for states of `state` values a column."""
+    return bool(_lib_fn("recurrent", "li_ssm_scan_layout", [c_int, c_int, c_void_p, c_void_p], c_int)(int(state), int(vdim), None, None))
+
+
+def causal_conv_silu(u: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor], tail: torch.Tensor, ctx, out: torch.Tensor) -> None:
+    """out[t, c] = silu(b[c] + sum_j w[c, j] u[t - (taps - 1 - j), c]) over each request's own tokens; what lies before
+    the step's portion comes from `tail` [slots, taps - 1, C] (zeros for a new request), which then takes the
+    request's last taps - 1 inputs.  u: float32 rows (a view with a row stride), the first C columns are read."""
+    _gpu(u, w, b, tail, out)
+    t, (c, taps) = out.shape[0], w.shape
+    _chk(u.dtype is torch.float32 and _rows_ok(u) and u.shape[0] == t and u.shape[1] >= c and out.dtype is torch.float32
+         and _rows_ok(out) and out.shape[1] == c, "causal_conv_silu: u, out")
+    _chk(w.dtype is torch.float32 and w.is_contiguous() and taps >= 1
+         and (b is None or (b.dtype is torch.float32 and b.numel() == c and b.is_contiguous())), "causal_conv_silu: w [C, taps], b [C] float32")
+    _chk(tail.dtype is torch.float32 and tail.is_contiguous() and tail.dim() == 3 and (taps == 1 or tail.shape[1:] == (taps - 1, c)),
+         "causal_conv_silu: tail [slots, taps - 1, C] float32")
+    _chk(ctx.num_tokens == t and int(ctx.host_state_slots.max(initial=0)) < tail.shape[0], "causal_conv_silu: batch")
+    if t:
+        _run("recurrent", "li_causal_conv_silu", u.data_ptr(), u.stride(0), c, taps, w.data_ptr(), 0 if b is None else b.data_ptr(),
+             tail.data_ptr(), ctx.seg_of_token.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(), ctx.state_slots.data_ptr(),
+             out.data_ptr(), out.stride(0), t, ctx.num_segments)
+
+
+def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d: torch.Tensor,
+             state: torch.Tensor, ctx, y: torch.Tensor, heads: int, vdim: int, n_state: int, groups: int, ws) -> None:
+    """The state-space recurrence over each request's tokens of the step, from and into `state`
+    [slots, heads, n_state, vdim] (float32):  S <- exp(-exp(a_log_h) dt) S + dt B x^T,  y = S^T C + d_h x,  with
+    dt = softplus(dt_raw + dt_bias_h).  xbc: float32 rows [x: heads * vdim | B: groups * n_state | C: groups * n_state];
+    dt: float32 rows [heads] (raw); y: float32 rows [heads * vdim].  All float32."""
+    _gpu(xbc, dt, dt_bias, a_log, d, state, y)
+    t = y.shape[0]
+    inner = heads * vdim
+    _chk(all(x.dtype is torch.float32 for x in (xbc, dt, dt_bias, a_log, d, state, y)), "ssm_scan: everything is float32")
+    _chk(_rows_ok(xbc) and xbc.shape == (t, inner + 2 * groups * n_state) and _rows_ok(dt) and dt.shape == (t, heads)
+         and _rows_ok(y) and y.shape == (t, inner), "ssm_scan: rows")
+    _chk(state.is_contiguous() and state.shape[1:] == (heads, n_state, vdim) and heads % groups == 0
+         and all(v.numel() == heads and v.is_contiguous() for v in (dt_bias, a_log, d)), "ssm_scan: state [slots, heads, N, vdim]")
+    _chk(ctx.num_tokens == t and int(ctx.host_state_slots.max(initial=0)) < state.shape[0], "ssm_scan: batch")
+    _chk(ssm_scan_takes(n_state, vdim), f"ssm_scan: no kernel for a state of {n_state} values a column (at most 256)")
+    if not t:
+        return
+    work, work_bytes = 0, 0
+    if ctx.max_q_len > SSM_CHUNK:
+        need = _lib_fn("recurrent", "li_ssm_scan_work_bytes", [c_int] * 6 + [c_void_p], c_long)(
+            t, ctx.num_segments, heads, vdim, n_state, SSM_CHUNK, None)
+        buf = ws.buffer("ssm_scan.work", ((int(need) + 3) // 4,), torch.float32)
+        work, work_bytes = buf.data_ptr(), buf.numel() * 4
+    _run("recurrent", "li_ssm_scan", xbc.data_ptr(), xbc.stride(0), dt.data_ptr(), dt.stride(0), dt_bias.data_ptr(), a_log.data_ptr(),
+         d.data_ptr(), state.data_ptr(), ctx.state_slots.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(), y.data_ptr(),
+         y.stride(0), heads, vdim, n_state, groups, SSM_CHUNK, t, ctx.num_segments, int(ctx.max_q_len), work, work_bytes)
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, out: torch.Tensor) -> None:
+    """out = weight * v / sqrt(mean over the group of v^2 + eps), v = y * silu(z), every one of `groups` equal runs of
+    columns by its own mean.  y, z float32 rows; out in either dtype."""
+    _gpu(y, z, weight, out)
+    t, n = out.shape
+    _chk(y.dtype is torch.float32 and z.dtype is torch.float32 and _rows_ok(y) and _rows_ok(z) and y.shape == (t, n) and z.shape == (t, n)
+         and _rows_ok(out) and out.dtype in _DT and weight.dtype is torch.float32 and weight.numel() == n and weight.is_contiguous()
+         and groups > 0 and n % groups == 0, "gated_group_norm: y, z [T, n] float32, weight [n], out [T, n]")
+    if t:
+        _run("recurrent", "li_gated_group_norm", y.data_ptr(), y.stride(0), z.data_ptr(), z.stride(0), weight.data_ptr(), float(eps),
+             out.data_ptr(), _DT[out.dtype], out.stride(0), t, n, int(groups))
+
+
+# --------------------------------------------------------------------------------------- routed feed-forward
+MOE_TILE_ROWS = 32       # rows of one expert that a block of the products takes
+
+
+def moe_max_tiles(tokens: int, top: int, experts: int) -> int:
+    """The most tiles a step can have: every expert's rows end in a tile that may not be full."""
+    pairs = tokens * top
+    return min(pairs, pairs // MOE_TILE_ROWS + experts)
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], gate_row: Optional[torch.Tensor],
+              idx: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor]) -> None:
+    """idx [T, top] int32: the experts with the largest logits x router^T + bias (float32 sums; the lower index wins a
+    tie); wt [T, top] float32: softmax over the chosen logits; gate [T] = sigmoid(x . gate_row) where a row is given."""
+    _gpu(x, router, bias, gate_row, idx, wt, gate)
+    t, k = x.shape
+    e, top = router.shape[0], idx.shape[1]
+    _chk(x.dtype in _DT and _rows_ok(x) and router.dtype in _DT and router.is_contiguous() and router.shape == (e, k)
+         and (bias is None or (bias.dtype is torch.float32 and bias.numel() == e and bias.is_contiguous())), "moe_route: x, router, bias")
+    _chk(idx.dtype is torch.int32 and idx.is_contiguous() and idx.shape == (t, top) and wt.dtype is torch.float32 and wt.is_contiguous()
+         and wt.shape == (t, top) and 1 <= top <= min(e, 64), "moe_route: idx, wt [T, top], top at most 64")
+    _chk((gate_row is None) == (gate is None) and (gate_row is None or (gate_row.dtype is router.dtype and gate_row.numel() == k
+         and gate_row.is_contiguous() and gate.dtype is torch.float32 and gate.numel() == t and gate.is_contiguous())), "moe_route: gate")
+    _chk((k + e) * 4 <= 60000, "moe_route: the row and the logits must fit 60 KB of LDS")
+    if t:
+        _run("moe", "li_moe_route", x.data_ptr(), _DT[x.dtype], x.stride(0), router.data_ptr(), _DT[router.dtype],
+             0 if bias is None else bias.data_ptr(), 0 if gate_row is None else gate_row.data_ptr(), idx.data_ptr(), wt.data_ptr(),
+             0 if gate is None else gate.data_ptr(), t, k, e, top)
+
+
+def moe_plan(idx: torch.Tensor, experts: int, plan: torch.Tensor, row_token: torch.Tensor, pair_row: torch.Tensor) -> int:
+    """Sorts the (token, choice) pairs by expert.  plan int32 [4 + 4 * max_tiles]: the number of tiles, then (expert,
+    first row, rows, 0) a tile; row_token [pairs]: the token of a sorted row; pair_row [pairs]: the row of a pair.
+    Returns max_tiles."""
+    _gpu(idx, plan, row_token, pair_row)
+    t, top = idx.shape
+    max_tiles = moe_max_tiles(t, top, experts)
+    _chk(all(x.dtype is torch.int32 and x.is_contiguous() for x in (idx, plan, row_token, pair_row))
+         and plan.numel() >= 4 + 4 * max_tiles and row_token.numel() >= t * top and pair_row.numel() >= t * top and experts <= 8000,
+         "moe_plan: int32 arrays of the step's sizes")
+    if t:
+        _run("moe", "li_moe_plan", idx.data_ptr(), t, top, experts, plan.data_ptr(), max_tiles, row_token.data_ptr(), pair_row.data_ptr())
+    return max_tiles
+
+
+def moe_linear(a: torch.Tensor, row_token: Optional[torch.Tensor], w: torch.Tensor, plan: torch.Tensor, max_tiles: int,
+               out: torch.Tensor, rows: int, act: int = 0) -> None:
+    """out[row] = act(W[expert of the row's tile] a[src(row)]) for the sorted rows of the plan; src(row) = row_token[row]
+    where given (rows gathered from tokens), else the row.  w [experts, n_out, K]; act 1: max(., 0)^2."""
+    _gpu(a, row_token, w, plan, out)
+    e, n_out, k = w.shape
+    _chk(a.dtype in _DT and _rows_ok(a) and a.shape[1] == k and w.dtype in _DT and w.is_contiguous() and out.dtype in _DT and _rows_ok(out)
+         and out.shape == (rows, n_out) and (w.dtype is torch.bfloat16 or (a.dtype is torch.float32 and out.dtype is torch.float32)),
+         "moe_linear: a [*, K], w [E, n_out, K], out [rows, n_out]")
+    _chk(plan.dtype is torch.int32 and plan.numel() >= 4 + 4 * max_tiles and (row_token is not None or a.shape[0] >= rows)
+         and (row_token is None or (row_token.dtype is torch.int32 and row_token.numel() >= rows)), "moe_linear: plan, rows")
+    if rows:
+        _run("moe", "li_moe_linear", a.data_ptr(), _DT[a.dtype], a.stride(0), 0 if row_token is None else row_token.data_ptr(),
+             w.data_ptr(), _DT[w.dtype], plan.data_ptr(), int(max_tiles), out.data_ptr(), _DT[out.dtype], out.stride(0), n_out, k, int(act))
+
+
+def moe_combine(x: torch.Tensor, yrows: torch.Tensor, pair_row: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor],
+                shared_out: Optional[torch.Tensor]) -> None:
+    """x[t] += sum_c wt[t, c] * yrows[pair_row[t * top + c]] (in the order of c) + gate[t] * shared_out[t]; float32."""
+    _gpu(x, yrows, pair_row, wt, gate, shared_out)
+    t, h = x.shape
+    top = wt.shape[1]
+    _chk(x.dtype is torch.float32 and _rows_ok(x) and yrows.dtype is torch.float32 and _rows_ok(yrows) and yrows.shape == (t * top, h)
+         and pair_row.dtype is torch.int32 and pair_row.numel() >= t * top and wt.dtype is torch.float32 and wt.is_contiguous()
+         and wt.shape[0] == t, "moe_combine: x [T, H], yrows [T * top, H], pair_row, wt")
+    _chk(shared_out is None or (shared_out.dtype is torch.float32 and _rows_ok(shared_out) and shared_out.shape == (t, h)
+                                and (gate is None or (gate.dtype is torch.float32 and gate.numel() == t))), "moe_combine: shared")
+    if t:
+        _run("moe", "li_moe_combine", x.data_ptr(), x.stride(0), yrows.data_ptr(), yrows.stride(0), pair_row.data_ptr(), wt.data_ptr(),
+             0 if gate is None else gate.data_ptr(), 0 if shared_out is None else shared_out.data_ptr(),
+             0 if shared_out is None else shared_out.stride(0), t, h, top)

@@ -7,6 +7,9 @@ from .norm import RMSNorm
 from .attention import GQAttention
 from .masked_attention import LatentAttention, MaskedAttention
 from .mlp import ReluSquaredMLP, SwiGLUMLP
+from .moe import RoutedReluSquaredMLP
+from .mamba2 import Mamba2Mixer
+from .diff_attention import DiffAttention
 from .block import PreNormBlock, SandwichBlock
 from .token_side import TokenSideInput
 from .inject import LoopEntry
@@ -16,4 +19,4 @@ __all__ = ["BatchNeeds", "Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed",
            "Part", "Runtime", "StateNeed", "needs_of",
            "build_part", "register_part", "Position", "RopeNeox", "Linear", "ResidualStream", "RMSNorm",
            "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding", "RopePairs", "BranchStream",
-           "MaskedAttention", "LatentAttention", "ReluSquaredMLP", "SandwichBlock", "TokenSideInput", "LoopEntry"]
+           "MaskedAttention", "LatentAttention", "RoutedReluSquaredMLP", "Mamba2Mixer", "DiffAttention", "ReluSquaredMLP", "SandwichBlock", "TokenSideInput", "LoopEntry"]

@@ -1,6 +1,6 @@
 """The pre-norm arrangement of a layer's parts
 (src/llaisys/models/qwen2.cpp:272-317): x += mixer(norm1(x)); x += ffn(norm2(x)).
-The residual stream x is float32; mixer and feed-forward add into it through
+A layer may lack the feed-forward (and its norm).  The residual stream x is float32; mixer and feed-forward add into it through
 the `ResidualStream` they are given."""
 from __future__ import annotations
 
@@ -14,9 +14,11 @@ class PreNormBlock(Block):
         super().__init__(spec, rt)
         self.norm1 = build_part("norm", parts["norm1"], rt)
         self.mixer = build_part("mixer", parts["mixer"], rt)
-        self.norm2 = build_part("norm", parts["norm2"], rt)
-        self.ffn = build_part("feed_forward", parts["feed_forward"], rt)
-        self._all = (self.norm1, self.mixer, self.norm2, self.ffn)
+        self.norm2 = self.ffn = None
+        if parts.get("feed_forward") is not None:
+            self.norm2 = build_part("norm", parts["norm2"], rt)
+            self.ffn = build_part("feed_forward", parts["feed_forward"], rt)
+        self._all = tuple(p for p in (self.norm1, self.mixer, self.norm2, self.ffn) if p is not None)
 
     @property
     def graph_safe(self):
@@ -47,10 +49,11 @@ class PreNormBlock(Block):
     def forward(self, stream, ctx, cache):
         xn = ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype)
         after = stream.next_norm                   # the norm that reads the stream after this block
-        stream.next_norm = self.norm2
+        stream.next_norm = self.norm2 if self.ffn is not None else after
         self.mixer.forward_prenorm(self.norm1, stream, xn, ctx, cache)
-        stream.next_norm = after
-        self.ffn.forward_prenorm(self.norm2, stream, xn, ctx)
+        if self.ffn is not None:
+            stream.next_norm = after
+            self.ffn.forward_prenorm(self.norm2, stream, xn, ctx)
         stream.next_norm = None
 
 

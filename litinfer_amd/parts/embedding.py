@@ -5,7 +5,13 @@ Embedding: x[t, :] = E[ids[t], :], a row copy without scaling
 Head: logits = xf Wout^T without bias (src/llaisys/models/qwen2.cpp:337), as
 float32; when tied, Wout is the embedding table itself (one buffer), and so it
 is when the configuration says untied but the checkpoint holds no head matrix
-(python/llaisys/models/qwen2.py:196-199)."""
+(python/llaisys/models/qwen2.py:196-199).
+
+Options that other designs use: the embedding may add a sinusoidal position vector
+(`sinusoid_base` b: column 2i gets sin(p b^(-2i/H)), column 2i+1 the cosine of the same
+angle; the frequencies are worked out once in float64 and rounded to float32, the angle is
+float(p) * f in float32); the head may scale its logits (`logit_scale`) and cap them
+(`softcap` c: c * tanh(logits / c)), in that order."""
 from __future__ import annotations
 
 import torch
@@ -26,16 +32,27 @@ class TokenEmbedding(Part):
         self.vocab = int(spec.args["vocab_size"])
         self.hidden = int(spec.args["hidden_size"])
         self.param = self.prefix + str(spec.args.get("param", "weight"))
+        self.sinusoid_base = float(spec.args.get("sinusoid_base") or 0.0)
+        if self.sinusoid_base < 0:
+            raise ValueError("embedding: the base of the position vector must be positive")
         self.table = None
+        self.freq = None
 
     def expected_params(self):
         return {self.param: ParamSpec((self.vocab, self.hidden))}
 
     def load_params(self, get):
         self.table = self.rt.matrix(get(self.param))
+        if self.sinusoid_base:
+            i = torch.arange((self.hidden + 1) // 2, dtype=torch.float64)
+            self.freq = self.rt.vector(torch.pow(torch.tensor(self.sinusoid_base, dtype=torch.float64), -2.0 * i / self.hidden))
 
-    def forward(self, ids, out, id_src=None, feedback=None):
+    def forward(self, ids, out, id_src=None, feedback=None, positions=None):
         ops.embedding(ids, self.table, out, id_src, feedback)
+        if self.freq is not None:
+            if positions is None:
+                raise ValueError("embedding: the position vector needs the tokens' positions")
+            ops.sinusoid_add(out, positions, self.freq)
         return out
 
 
@@ -52,6 +69,10 @@ class LinearHead(Part):
         # untied by the configuration, but no matrix stored: use the table, as the reference does
         self.tie_if_absent = bool(spec.args.get("tie_if_absent", False))
         self.param = self.prefix + str(spec.args.get("param", "weight"))
+        self.logit_scale = float(spec.args.get("logit_scale") if spec.args.get("logit_scale") is not None else 1.0)
+        self.softcap = float(spec.args.get("softcap") or 0.0)
+        if self.softcap < 0:
+            raise ValueError("head: the cap of the logits must not be negative")
         self.proj = None
 
     def expected_params(self):
@@ -72,7 +93,10 @@ class LinearHead(Part):
             self.proj = Linear(self.rt, w)
 
     def forward(self, xn, out, ws):
-        return self.proj(xn, out, ws=ws)
+        self.proj(xn, out, ws=ws)
+        if self.logit_scale != 1.0 or self.softcap:
+            ops.scale_softcap(out, self.logit_scale, self.softcap)
+        return out
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)

@@ -1,0 +1,106 @@
+"""A routed feed-forward: `experts` small feed-forwards of which every token uses `top`, and an optional shared
+one that every token uses.
+
+Router: logits = xn Wr^T + br in float32; the `top` largest are chosen (the lower index wins a tie) and weighted
+by the softmax over the chosen logits alone.  An expert is Wdown act(Wup xn) with act = max(., 0)^2, no biases.
+The shared expert has the same form with a width of its own; its output is multiplied by sigmoid(wg . xn), one
+number a token, where a gate row is given.  The output is the weighted sum, added to the stream in float32.
+
+On the device: one kernel routes (logits, choice, weights and the shared gate), one sorts the step's (token,
+choice) pairs by expert and cuts them into tiles of rows, the two products run tile by tile against the
+tile's expert (the activation is the first one's epilogue), and one kernel adds the weighted rows and the gated
+shared output into the stream, in the order of the choices.  No number returns to the host, so a decoding step
+can be recorded.  The experts' matrices are bound as two tensors [experts, ff, hidden] and [experts, hidden, ff].
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import ParamSpec
+from .base import BatchNeeds, FeedForward, register_part
+from .linear import Linear
+
+
+class RoutedReluSquaredMLP(FeedForward):
+    graph_safe = True
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        a = spec.args
+        self.hidden = int(a["hidden_size"])
+        self.experts = int(a["experts"])
+        self.top = int(a["top"])
+        self.inter = int(a["intermediate_size"])
+        self.shared_inter = int(a.get("shared_intermediate_size") or 0)
+        self.shared_gate = bool(a.get("shared_gate", True)) and self.shared_inter > 0
+        if min(self.hidden, self.experts, self.top, self.inter) <= 0 or self.top > self.experts:
+            raise ValueError(f"routed feed-forward: {self.top} of {self.experts} experts of width {self.inter}")
+        if self.top > 64:
+            raise ValueError("routed feed-forward: the router kernel picks at most 64 experts a token")
+        self.names = {"expert": "e{}.", "up": "up", "down": "down", "router": "router", "router_bias": "router.b",
+                      "shared": "shared.", "shared_gate": "sg", **(a.get("names") or {})}
+        self.w_up = self.w_down = self.router = self.router_b = self.gate_row = self.shared_up = self.shared_down = None
+
+    def _expert(self, e: int, which: str) -> str:
+        return self.prefix + self.names["expert"].format(e) + self.names[which]
+
+    def expected_params(self):
+        p, n = self.prefix, self.names
+        out = {p + n["router"]: ParamSpec((self.experts, self.hidden)),
+               p + n["router_bias"]: ParamSpec((self.experts,), init="zeros")}
+        for e in range(self.experts):
+            out[self._expert(e, "up")] = ParamSpec((self.inter, self.hidden))
+            out[self._expert(e, "down")] = ParamSpec((self.hidden, self.inter))
+        if self.shared_inter:
+            s = p + n["shared"]
+            out[s + n["up"]] = ParamSpec((self.shared_inter, self.hidden))
+            out[s + n["down"]] = ParamSpec((self.hidden, self.shared_inter))
+            if self.shared_gate:
+                out[s + n["shared_gate"]] = ParamSpec((1, self.hidden))
+        return out
+
+    def batch_needs(self):
+        return BatchNeeds(row_tile=self.shared_down.row_tile() if self.shared_down is not None else 1)
+
+    def load_params(self, get):
+        p, n = self.prefix, self.names
+        self.w_up = self.rt.matrix(torch.stack([get(self._expert(e, "up")) for e in range(self.experts)]))
+        self.w_down = self.rt.matrix(torch.stack([get(self._expert(e, "down")) for e in range(self.experts)]))
+        self.router = self.rt.matrix(get(p + n["router"]))
+        self.router_b = self.rt.vector(get(p + n["router_bias"]))
+        if self.shared_inter:
+            s = p + n["shared"]
+            self.shared_up = Linear(self.rt, get(s + n["up"]))
+            self.shared_down = Linear(self.rt, get(s + n["down"]))
+            if self.shared_gate:
+                self.gate_row = self.rt.matrix(get(s + n["shared_gate"]).reshape(-1))
+
+    def forward(self, xn, residual, ctx):
+        t, top, ws = xn.shape[0], self.top, ctx.ws
+        pairs = t * top
+        idx = ws.buffer("moe.idx", (t, top), torch.int32)
+        wt = ws.buffer("moe.wt", (t, top), torch.float32)
+        gate = ws.buffer("moe.gate", (t,), torch.float32) if self.gate_row is not None else None
+        ops.moe_route(xn, self.router, self.router_b, self.gate_row, idx, wt, gate)
+        max_tiles = ops.moe_max_tiles(t, top, self.experts)
+        plan = ws.buffer("moe.plan", (4 + 4 * max_tiles,), torch.int32)
+        row_token = ws.buffer("moe.row_token", (pairs,), torch.int32)
+        pair_row = ws.buffer("moe.pair_row", (pairs,), torch.int32)
+        ops.moe_plan(idx, self.experts, plan, row_token, pair_row)
+        h = ws.buffer("moe.h", (pairs, self.inter), self.rt.dtype)
+        ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=1)
+        yrows = ws.buffer("moe.y", (pairs, self.hidden), torch.float32)
+        ops.moe_linear(h, None, self.w_down, plan, max_tiles, yrows, pairs)
+        shared = None
+        if self.shared_inter:
+            u = ws.buffer("mlp.up32", (t, self.shared_inter), torch.float32)
+            self.shared_up(xn, u, ws=ws)
+            hs = ws.buffer("mlp.h", (t, self.shared_inter), self.rt.dtype)
+            ops.relu_squared(u, hs)
+            shared = ws.buffer("moe.shared", (t, self.hidden), torch.float32)
+            self.shared_down(hs, shared, ws=ws)
+        ops.moe_combine(residual.tensor(), yrows, pair_row, wt, gate, shared)
+
+
+register_part("feed_forward", "routed_relu2", RoutedReluSquaredMLP)

@@ -1,6 +1,8 @@
 """RMSNorm: y = w * x / sqrt(mean(x^2) + eps), computed in 32-bit
 (src/ops/rms_norm/op.cpp:13-23: eps inside the root, the weight multiplies
-directly)."""
+directly).  With `offset` (an argument, default 0) the stored tensor lies around
+zero and the weight is offset + stored: y = (offset + w) * x / sqrt(...); the sum
+is made once, in float32, when the tensor is bound."""
 from __future__ import annotations
 
 from ..kernels import ops
@@ -18,13 +20,16 @@ class RMSNorm(Norm):
         if self.eps < 0:
             raise ValueError(f"rmsnorm: eps must not be negative, found {self.eps}")
         self.param = self.prefix + str(spec.args.get("param", "weight"))     # the tensor's name behind the prefix
+        self.offset = float(spec.args.get("offset") or 0.0)
         self.weight = None
 
     def expected_params(self):
-        return {self.param: ParamSpec((self.size,), init="one_plus_normal")}
+        return {self.param: ParamSpec((self.size,), init="normal" if self.offset else "one_plus_normal")}
 
     def load_params(self, get):
         self.weight = self.rt.vector(get(self.param))
+        if self.offset:
+            self.weight = (self.weight + self.offset).contiguous()
 
     def forward(self, x, out):
         ops.rmsnorm(x, self.weight, self.eps, out)
