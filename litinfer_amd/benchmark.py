@@ -738,9 +738,31 @@ def tovasun_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, obje
             "loop": {"start": 1, "stop": 3, "times": 2} if layers >= 4 else None, "token_side": {"dim": side}}
 
 
+SOGENEX_SIZES = {         # state-space heads x columns, state, groups; attention heads (two maps each), kv heads, key size, value size;
+    # experts, chosen, expert width, shared width: the chosen experts and the shared one together are as wide as the dense feed-forward
+    "1.5b": (48, 64, 128, 8, 12, 2, 64, 128, 16, 2, 2240, 4480),
+    "7b": (112, 64, 128, 8, 28, 4, 64, 128, 16, 2, 4736, 9472),
+}
+
+
+def sogenex_config(size: str, layers: int, vocab: int = 32000) -> Dict[str, object]:
+    """A Sogenex model at the width of a Qwen2 family member: state-space layers with every third one a windowed
+    differential attention, each with a routed feed-forward whose active width is the dense one's."""
+    width = DESIGN_SIZES[size][0]
+    sh, sv, sn, sg, ah, akv, ad, av, ne, top, eff, sff = SOGENEX_SIZES[size]
+    mlp = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": ne, "top": top}, "shared": {"ff": sff}}
+    ssm = {"type": "mamba2", "mlp": mlp,
+           "mixer": {"heads": sh, "vdim": sv, "state": sn, "groups": sg, "conv": 4, "norm_groups": sg}}
+    attn = {"type": "attention", "mlp": mlp,
+            "mixer": {"heads": ah, "kv_heads": akv, "dim": ad, "vdim": av, "diff": 0.3, "scale": ad ** -0.5,
+                      "mask": {"size": DESIGN_WINDOW}}}
+    return {"architecture": "Sogenex", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+            "logit_softcap": 30.0, "layers": [attn if i % 3 == 1 else ssm for i in range(layers)]}
+
+
 def compare_designs(a) -> Dict[str, object]:
-    """Prefill and decode throughput of Tovasun beside Qwen2 at the same width, heads, feed-forward width,
-    window and number of layer runs (random weights, random cache content)."""
+    """Prefill and decode throughput of a second design (`--design`: Tovasun or Sogenex) beside Qwen2 at the same
+    width, heads, (active) feed-forward width, window and number of layer runs (random weights, random cache content)."""
     import numpy as np
     import torch
     from .engine import Engine, StepEntry
@@ -750,13 +772,14 @@ def compare_designs(a) -> Dict[str, object]:
     batches = (1, a.batch, 64)
     for size in sizes:
         layers = a.layers or 6
-        tcfg = tovasun_config(size, layers)
-        runs = layers + (2 if tcfg["loop"] else 0)
+        design = getattr(a, "design", None) or "tovasun"
+        tcfg = sogenex_config(size, layers) if design == "sogenex" else tovasun_config(size, layers)
+        runs = layers + (2 if tcfg.get("loop") else 0)
         width, heads, kv, dim, ff = DESIGN_SIZES[size][:5]
         qcfg = dict(SHAPES[size], num_hidden_layers=runs, vocab_size=32000, use_sliding_window=True,
                     sliding_window=DESIGN_WINDOW, max_window_layers=0, max_position_embeddings=8192)
         res = {}
-        for name, cfg, vocab in (("tovasun", tcfg, tcfg["vocab"]), ("qwen2", qcfg, qcfg["vocab_size"])):
+        for name, cfg, vocab in ((design, tcfg, tcfg["vocab"]), ("qwen2", qcfg, qcfg["vocab_size"])):
             eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
                                      num_pages=(64 * (DESIGN_WINDOW + 64) + 2 * PREFILL_TOKENS) // PAGE, max_seqs=65)
             for g in eng.cache.groups:
@@ -804,16 +827,17 @@ def compare_designs(a) -> Dict[str, object]:
             log(f"{size} {name}: {r}")
             del eng
             torch.cuda.empty_cache()
-        res["tovasun_over_qwen2"] = {k: round(res["tovasun"][k] / res["qwen2"][k], 3)
-                                     for k in res["qwen2"] if k.endswith("tok_s")}
+        res[f"{design}_over_qwen2"] = {k: round(res[design][k] / res["qwen2"][k], 3)
+                                       for k in res["qwen2"] if k.endswith("tok_s")}
         out[size] = res
     first = out[sizes[0]]
-    return {"metric": f"decode tok/s (Tovasun at the Qwen2-{sizes[0]} layer sizes, batch {a.batch}, window {DESIGN_WINDOW})",
-            "value": first["tovasun"][f"decode_b{a.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
-            "warmup": a.warmup, "ms_per_step": first["tovasun"][f"decode_b{a.batch}_ms"], "higher_is_better": True,
+    title = design.capitalize()
+    return {"metric": f"decode tok/s ({title} at the Qwen2-{sizes[0]} layer sizes, batch {a.batch}, window {DESIGN_WINDOW})",
+            "value": first[design][f"decode_b{a.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
+            "warmup": a.warmup, "ms_per_step": first[design][f"decode_b{a.batch}_ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": a.dtype,
             "data": "synthetic: seeded random token ids, random weights N(0, 0.02), random cache content",
-            "config": {"model": "Tovasun beside Qwen2 at equal layer sizes", "global_batch": a.batch,
+            "config": {"model": f"{title} beside Qwen2 at equal layer sizes", "global_batch": a.batch,
                        "seq_len": 2 * DESIGN_WINDOW, "prefill_tokens": PREFILL_TOKENS, "page_size": PAGE,
                        "parallelism": "none (1 GPU)"},
             "designs": out}
@@ -830,6 +854,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep", "designs"])
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES),
                     help="sweep: the member of the family whose layer sizes are taken (7b); designs: 1.5b or 7b (both)")
+    ap.add_argument("--design", default="tovasun", choices=["tovasun", "sogenex"],
+                    help="designs: the design that is set beside Qwen2")
     ap.add_argument("--page-order-seed", type=int, default=0,
                     help="headline: the cache's pages are handed out in a shuffled order, as a pool that has served requests "
                          "does (negative: in the order of their numbers; a request's keys then lie in one piece, and "
