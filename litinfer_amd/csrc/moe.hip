@@ -10,22 +10,49 @@
 // ------------------------------------------------------------------------------------------------ router
 // One block a token.  logits[e] = b[e] + sum_k W[e, k] x[k] in float32 (a wave an expert, in turns); the `top`
 // largest (the lower index wins a tie), weights = softmax over the chosen logits.  gate[t] = sigmoid(wg . x).
-template <typename TX, typename TW>
-__global__ __launch_bounds__(256) void moe_route_kernel(const TX* __restrict__ x, long x_stride, const TW* __restrict__ wr,
-                                                        const float* __restrict__ br, const TW* __restrict__ wg,
-                                                        int* __restrict__ idx, float* __restrict__ wt, float* __restrict__ gate,
-                                                        int K, int E, int top) {
-    extern __shared__ float sm[];                      // [K] the row, [E] the logits
+template <typename T> struct RouteVec;
+template <> struct RouteVec<float> { static constexpr int N = 4; };
+template <> struct RouteVec<bf16_t> { static constexpr int N = 8; };
+
+// 16 bytes of a matrix row against the row in LDS
+__device__ __forceinline__ float route_dot16(const float* p, const float* xs) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    return fmaf(v.x, xs[0], fmaf(v.y, xs[1], fmaf(v.z, xs[2], v.w * xs[3])));
+}
+__device__ __forceinline__ float route_dot16(const bf16_t* p, const float* xs) {
+    const uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t u[4] = {r.x, r.y, r.z, r.w};
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        s = fmaf(__uint_as_float(u[i] << 16), xs[2 * i], s);
+        s = fmaf(__uint_as_float(u[i] & 0xffff0000u), xs[2 * i + 1], s);
+    }
+    return s;
+}
+
+template <typename TX, typename TW, int NT>
+__global__ __launch_bounds__(NT) void moe_route_kernel(const TX* __restrict__ x, long x_stride, const TW* __restrict__ wr,
+                                                       const float* __restrict__ br, const TW* __restrict__ wg,
+                                                       int* __restrict__ idx, float* __restrict__ wt, float* __restrict__ gate,
+                                                       int K, int E, int top, int vec) {
+    extern __shared__ __align__(16) float sm[];        // [K] the row, [E] the logits
     float* xs = sm;
-    float* lg = sm + K;
+    float* lg = sm + ((K + 3) & ~3);
     const int t = blockIdx.x, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const TX* row = x + (size_t)t * x_stride;
-    for (int k = threadIdx.x; k < K; k += 256) xs[k] = load_as_float(row + k);
+    for (int k = threadIdx.x; k < K; k += NT) xs[k] = load_as_float(row + k);
     __syncthreads();
-    for (int e = w; e < E + (wg ? 1 : 0); e += 4) {
+    constexpr int VE = RouteVec<TW>::N;
+    for (int e = w; e < E + (wg ? 1 : 0); e += NT / 64) {
         const TW* wrow = e < E ? wr + (size_t)e * K : wg;
         float s = 0.f;
-        for (int k = lane; k < K; k += 64) s = fmaf(load_as_float(wrow + k), xs[k], s);
+        if (vec) {                                     // 16 bytes a lane and turn, several turns on their way
+#pragma unroll 4
+            for (int i = lane; i < K / VE; i += 64) s += route_dot16(wrow + (size_t)i * VE, xs + i * VE);
+        } else {
+            for (int k = lane; k < K; k += 64) s = fmaf(load_as_float(wrow + k), xs[k], s);
+        }
         s = wave_sum(s);
         if (lane == 0) {
             if (e < E) lg[e] = s + (br ? br[e] : 0.f);
@@ -65,14 +92,22 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const TX* __restrict__ x
 
 extern "C" int li_moe_route(const void* x, int x_dtype, long x_stride, const void* wr, int w_dtype, const float* br, const void* wg,
                             int* idx, float* wt, float* gate, int T, int K, int E, int top, hipStream_t stream) {
-    if (T <= 0 || K <= 0 || E <= 0 || top <= 0 || top > E || top > 64 || x_stride < K || (size_t)(K + E) * 4 > 60000 || (wg && !gate))
+    if (T <= 0 || K <= 0 || E <= 0 || top <= 0 || top > E || top > 64 || x_stride < K || (size_t)(K + E + 4) * 4 > 60000 || (wg && !gate))
         return LI_ERR_SIZE;
-    const size_t lds = (size_t)(K + E) * 4;
-#define MR(TX, TW) moe_route_kernel<TX, TW><<<T, 256, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top)
-    if (x_dtype == LI_F32 && w_dtype == LI_F32) MR(float, float);
-    else if (x_dtype == LI_BF16 && w_dtype == LI_BF16) MR(bf16_t, bf16_t);
-    else if (x_dtype == LI_BF16 && w_dtype == LI_F32) MR(bf16_t, float);
-    else if (x_dtype == LI_F32 && w_dtype == LI_BF16) MR(float, bf16_t);
+    const size_t lds = (size_t)(((K + 3) & ~3) + E) * 4;
+    // whole 16-byte pieces of every matrix row (the gate row included)
+    const int ve = w_dtype == LI_F32 ? 4 : 8;
+    const int vec = K % ve == 0 && ((uintptr_t)wr % 16) == 0 && (!wg || ((uintptr_t)wg % 16) == 0);
+    // few tokens: sixteen waves share a token's experts, so that a wave has one or two rows to go through
+#define MR(TX, TW)                                                                                                                \
+    {                                                                                                                             \
+        if (T <= 128) moe_route_kernel<TX, TW, 1024><<<T, 1024, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top, vec); \
+        else moe_route_kernel<TX, TW, 256><<<T, 256, lds, stream>>>((const TX*)x, x_stride, (const TW*)wr, br, (const TW*)wg, idx, wt, gate, K, E, top, vec);           \
+    }
+    if (x_dtype == LI_F32 && w_dtype == LI_F32) MR(float, float)
+    else if (x_dtype == LI_BF16 && w_dtype == LI_BF16) MR(bf16_t, bf16_t)
+    else if (x_dtype == LI_BF16 && w_dtype == LI_F32) MR(bf16_t, float)
+    else if (x_dtype == LI_F32 && w_dtype == LI_BF16) MR(float, bf16_t)
     else return LI_ERR_DTYPE;
 #undef MR
     return li_launch_status();
@@ -249,18 +284,154 @@ __global__ __launch_bounds__(256) void moe_linear_mfma_kernel(const TA* __restri
     }
 }
 
+// The wider form, for K a multiple of 32: a wave takes the tile's 32 rows and 128 outputs (four accumulators that
+// share the rows' operand), K in steps of 32 with the next step's ten loads asked for before this step's eight
+// matrix products.  KSPLIT = 1: the four waves of a block take 512 outputs side by side (many rows: a prompt).
+// KSPLIT = 4: they take the same 128 outputs and a quarter of K each and add up through LDS, so that the few tiles
+// of a decoding step, each of which streams its expert's whole matrix, are spread over four times the waves.
+template <typename TA>
+__device__ __forceinline__ void moe_load_rows(moe_frag8& f, const TA* p) {
+    if constexpr (sizeof(TA) == 2) {
+        f.raw = *reinterpret_cast<const uint4*>(p);
+    } else {
+        const float4 u = *reinterpret_cast<const float4*>(p);
+        const float4 v = *reinterpret_cast<const float4*>(p + 4);
+        f.w[0] = pack2_bf16(u.x, u.y); f.w[1] = pack2_bf16(u.z, u.w);
+        f.w[2] = pack2_bf16(v.x, v.y); f.w[3] = pack2_bf16(v.z, v.w);
+    }
+}
+
+template <typename TA, typename TO, int KSPLIT>
+__global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restrict__ a, long a_stride, const int* __restrict__ row_token,
+                                                              const bf16_t* __restrict__ w, const int* __restrict__ plan,
+                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act,
+                                                              int max_tiles) {
+    int tile = blockIdx.x, cb = blockIdx.y;
+    if (KSPLIT == 1) {
+        // Many tiles: the grid is one row of blocks, which the chip deals out to its eight XCDs in turn.  Eight tiles
+        // that follow each other (mostly rows of one expert) against the same columns go to ONE XCD, next to each other
+        // in time, so that the expert's matrix comes into that XCD's L2 once for them and not once for each XCD.
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        const int item = (((idx >> 3) << 3) + xcd) * 8 + (idx & 7);
+        const int tiles = max_tiles;
+        cb = item / tiles;
+        tile = item % tiles;
+    }
+    if (tile >= plan[0]) return;
+    const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ql = lane & 31, h2 = lane >> 5;
+    const int j0 = (KSPLIT == 1 ? cb * 4 + wv : cb) * 128;
+    if (KSPLIT == 1 && j0 >= n_out) return;
+    int nf = (n_out - j0) / 32;                        // column fragments of 32 that exist (n_out is a multiple of 32)
+    if (nf > 4) nf = 4;
+    int k0 = 0, k1 = K;
+    if (KSPLIT > 1) {
+        const int per = ((K / 32 + KSPLIT - 1) / KSPLIT) * 32;
+        k0 = wv * per;
+        k1 = k0 + per < K ? k0 + per : K;
+    }
+    const int r = r0 + (ql < nr ? ql : 0);
+    const TA* arow = a + (size_t)(row_token ? row_token[r] : r) * a_stride + 8 * h2;
+    const bf16_t* mrow[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) mrow[f] = w + ((size_t)e * n_out + j0 + 32 * (f < nf ? f : 0) + ql) * K + 8 * h2;
+    moe_f32x16 acc[4];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[f][i] = 0.f;
+    moe_frag8 ca[2], cw[4][2], na[2], nw[4][2];
+    if (k0 < k1) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            moe_load_rows<TA>(ca[s2], arow + k0 + 16 * s2);
+#pragma unroll
+            for (int f = 0; f < 4; ++f) cw[f][s2].raw = *reinterpret_cast<const uint4*>(mrow[f] + k0 + 16 * s2);
+        }
+    }
+    for (int k = k0; k < k1; k += 32) {
+        const int kn = k + 32 < k1 ? k + 32 : k;       // (the last turn asks for its own step again: no branch around the loads)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            moe_load_rows<TA>(na[s2], arow + kn + 16 * s2);
+#pragma unroll
+            for (int f = 0; f < 4; ++f) nw[f][s2].raw = *reinterpret_cast<const uint4*>(mrow[f] + kn + 16 * s2);
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int f = 0; f < 4; ++f) acc[f] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cw[f][s2].v, ca[s2].v, acc[f], 0, 0, 0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            ca[s2] = na[s2];
+#pragma unroll
+            for (int f = 0; f < 4; ++f) cw[f][s2] = nw[f][s2];
+        }
+    }
+    int f_lo = 0, f_hi = nf;
+    if (KSPLIT > 1) {
+        // the four waves' sums meet in LDS; wave f then owns column fragment f
+        __shared__ float red[KSPLIT][4][16][64];
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) red[wv][f][i][lane] = acc[f][i];
+        __syncthreads();
+        if (wv >= nf) return;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float t = 0.f;
+#pragma unroll
+            for (int src = 0; src < KSPLIT; ++src) t += red[src][wv][i][lane];
+            acc[0][i] = t;
+        }
+        f_lo = wv;
+        f_hi = wv + 1;
+    }
+    if (ql >= nr) return;
+    TO* orow = out + (size_t)(r0 + ql) * out_stride + j0;
+    for (int f = f_lo; f < f_hi; ++f) {
+        const moe_f32x16 c = KSPLIT > 1 ? acc[0] : (f == 0 ? acc[0] : f == 1 ? acc[1] : f == 2 ? acc[2] : acc[3]);
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {               // registers 4 rg .. 4 rg + 3: outputs 32 f + 8 rg + 4 h2 ..
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i] = c[4 * rg + i];
+                if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
+            }
+            TO* dst = orow + 32 * f + 8 * rg + 4 * h2;
+            if constexpr (sizeof(TO) == 2) {
+                uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
+                d2[0] = pack2_bf16(v[0], v[1]);
+                d2[1] = pack2_bf16(v[2], v[3]);
+            } else {
+                *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+            }
+        }
+    }
+}
+
 extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const int* row_token, const void* w, int w_dtype,
                              const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act,
                              hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || out_stride < n_out || act < 0 || act > 1) return LI_ERR_SIZE;
     if (w_dtype == LI_BF16 && K % 16 == 0 && n_out % 32 == 0 && a_stride % 8 == 0 && out_stride % 4 == 0 &&
         ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0 && (a_dtype == LI_BF16 || a_dtype == LI_F32)) {
+        // few tiles (a decoding step: each streams its expert's whole matrix): K in quarters over a block's waves
+        const bool wide = K % 32 == 0, split = wide && max_tiles <= 128 && K >= 256;
         const dim3 grid(max_tiles, (n_out + 127) / 128);
-#define MM(TA, TO) moe_linear_mfma_kernel<TA, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act)
-        if (a_dtype == LI_BF16 && out_dtype == LI_BF16) MM(bf16_t, bf16_t);
-        else if (a_dtype == LI_BF16 && out_dtype == LI_F32) MM(bf16_t, float);
-        else if (a_dtype == LI_F32 && out_dtype == LI_BF16) MM(float, bf16_t);
-        else if (a_dtype == LI_F32 && out_dtype == LI_F32) MM(float, float);
+        const dim3 line((unsigned)((((long)max_tiles * ((n_out + 511) / 512) + 63) / 64) * 64));       // whole rounds of eight tiles over eight XCDs
+#define MM(TA, TO)                                                                                                                 \
+    {                                                                                                                              \
+        if (split) moe_linear_wide_kernel<TA, TO, 4><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, max_tiles); \
+        else if (wide) moe_linear_wide_kernel<TA, TO, 1><<<line, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, max_tiles); \
+        else moe_linear_mfma_kernel<TA, TO><<<grid, 256, 0, stream>>>((const TA*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act); \
+    }
+        if (a_dtype == LI_BF16 && out_dtype == LI_BF16) MM(bf16_t, bf16_t)
+        else if (a_dtype == LI_BF16 && out_dtype == LI_F32) MM(bf16_t, float)
+        else if (a_dtype == LI_F32 && out_dtype == LI_BF16) MM(float, bf16_t)
+        else if (a_dtype == LI_F32 && out_dtype == LI_F32) MM(float, float)
         else return LI_ERR_DTYPE;
 #undef MM
         return li_launch_status();

@@ -194,6 +194,145 @@ __global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_kernel(
     }
 }
 
+// The same recurrence with FOUR neighbouring columns a lane (head sizes that are multiples of 4): lane = quad * NS +
+// slice holds NR state values of each of its four columns.  A value of B_t or C_t read from LDS then serves four
+// state elements instead of one, and the state comes from and goes to memory in 16-byte pieces.  A wave is 256 / NS
+// columns of one head.  Modes, chunks and blocks as above.
+template <int NR, int NS, int MODE>
+__global__ __launch_bounds__(64 * SSM_WAVES) void ssm_scan_quad_kernel(
+    const float* __restrict__ xbc, long xbc_stride, const float* __restrict__ dt_raw, long dt_stride,
+    const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ Dw,
+    float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ q_start, const int* __restrict__ q_len,
+    const int* __restrict__ chunk_seg, const int* __restrict__ chunk_idx, float* __restrict__ carry, float* __restrict__ decay,
+    float* __restrict__ y, long y_stride, int heads, int vdim, int N, int G, int Q) {
+    constexpr int NP = NR * NS, PW = 256 / NS;
+    extern __shared__ __align__(16) float lds[];
+    float* sB = lds;                                   // [SSM_TB][NP]
+    float* sC = sB + SSM_TB * NP;                      // [SSM_TB][NP]
+    float* sX = sC + SSM_TB * NP;                      // [SSM_WAVES][SSM_TB][PW]
+    float* sDt = sX + SSM_WAVES * SSM_TB * PW;         // [SSM_WAVES][SSM_TB]
+    float* sA = sDt + SSM_WAVES * SSM_TB;              // [SSM_WAVES][SSM_TB]
+    const int bx = blockIdx.x;
+    const int seg = chunk_seg ? chunk_seg[bx] : bx;
+    if (seg < 0) return;
+    const int c = chunk_seg ? chunk_idx[bx] : 0;
+    const int L = q_len[seg], first = c * Q;
+    if (first >= L) return;
+    const int ntok = (L - first < Q) ? L - first : Q;
+    const bool last = first + ntok >= L;
+    if (MODE == 1 && last) return;
+    const int t0 = q_start[seg] + first;
+    const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
+    const int g = blockIdx.y / ublocks, ub = blockIdx.y % ublocks;
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int unit = ub * SSM_WAVES + w;
+    const bool active = unit < U;
+    const int head = g * hpg + (active ? unit / PS : 0), pbase = active ? (unit % PS) * PW : 0;
+    const int pq = lane / NS, s = lane % NS, p = pbase + 4 * pq;        // the first of the lane's four columns
+    const bool cols = p < vdim;                                         // (vdim is a multiple of 4: all four or none)
+    const int inner = heads * vdim;
+    const size_t hoff = (size_t)head * N * vdim;
+    float4 S[NR];
+    if (MODE == 0 && active) {
+        const float* src = chunk_seg ? carry + (size_t)bx * heads * N * vdim + hoff
+                                     : state + (size_t)slots[seg] * heads * N * vdim + hoff;
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int n = s * NR + r;
+            S[r] = (n < N && cols) ? *reinterpret_cast<const float4*>(src + (size_t)n * vdim + p) : float4{0.f, 0.f, 0.f, 0.f};
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) S[r] = float4{0.f, 0.f, 0.f, 0.f};
+    }
+    float prod = 1.f;
+    const float Dh = (MODE == 0 && active) ? Dw[head] : 0.f;
+    for (int b0 = 0; b0 < ntok; b0 += SSM_TB) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < SSM_TB * NP; i += 64 * SSM_WAVES) {
+            const int tt = i / NP, n = i % NP;
+            const bool ok = b0 + tt < ntok && n < N;
+            const float* row = xbc + (size_t)(t0 + b0 + tt) * xbc_stride + inner + (size_t)g * N + n;
+            sB[i] = ok ? row[0] : 0.f;
+            sC[i] = ok ? row[(size_t)G * N] : 0.f;
+        }
+        if (active) {
+            for (int i = lane; i < SSM_TB * PW; i += 64) {
+                const int tt = i / PW, pp = pbase + i % PW;
+                const bool ok = b0 + tt < ntok && pp < vdim;
+                sX[(w * SSM_TB + tt) * PW + i % PW] = ok ? xbc[(size_t)(t0 + b0 + tt) * xbc_stride + (size_t)head * vdim + pp] : 0.f;
+            }
+            if (lane < SSM_TB) {
+                const bool ok = b0 + lane < ntok;
+                const float d = ok ? softplus_f32(dt_raw[(size_t)(t0 + b0 + lane) * dt_stride + head] + dt_bias[head]) : 0.f;
+                sDt[w * SSM_TB + lane] = d;
+                sA[w * SSM_TB + lane] = expf(-expf(A_log[head]) * d);
+            }
+        }
+        __syncthreads();
+        if (!active) continue;
+        const int nt = (ntok - b0 < SSM_TB) ? ntok - b0 : SSM_TB;
+        for (int tt = 0; tt < nt; ++tt) {
+            const float a = sA[w * SSM_TB + tt], dtv = sDt[w * SSM_TB + tt];
+            const float4 xv = *reinterpret_cast<const float4*>(sX + (w * SSM_TB + tt) * PW + 4 * pq);
+            const float4 dx = float4{dtv * xv.x, dtv * xv.y, dtv * xv.z, dtv * xv.w};
+            const float4* Bp = reinterpret_cast<const float4*>(sB + tt * NP + s * NR);
+            const float4* Cp = reinterpret_cast<const float4*>(sC + tt * NP + s * NR);
+            float4 yv = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int r4 = 0; r4 < NR / 4; ++r4) {
+                const float4 bv = Bp[r4];
+                const float bs[4] = {bv.x, bv.y, bv.z, bv.w};
+                float cs[4] = {0.f, 0.f, 0.f, 0.f};
+                if (MODE == 0) { const float4 cv = Cp[r4]; cs[0] = cv.x; cs[1] = cv.y; cs[2] = cv.z; cs[3] = cv.w; }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float4& st = S[4 * r4 + j];
+                    st.x = fmaf(a, st.x, bs[j] * dx.x);
+                    st.y = fmaf(a, st.y, bs[j] * dx.y);
+                    st.z = fmaf(a, st.z, bs[j] * dx.z);
+                    st.w = fmaf(a, st.w, bs[j] * dx.w);
+                    if (MODE == 0) {
+                        yv.x = fmaf(st.x, cs[j], yv.x);
+                        yv.y = fmaf(st.y, cs[j], yv.y);
+                        yv.z = fmaf(st.z, cs[j], yv.z);
+                        yv.w = fmaf(st.w, cs[j], yv.w);
+                    }
+                }
+            }
+            if (MODE == 0) {
+#pragma unroll
+                for (int o = 1; o < NS; o <<= 1) {
+                    yv.x += __shfl_xor(yv.x, o, LI_WAVE);
+                    yv.y += __shfl_xor(yv.y, o, LI_WAVE);
+                    yv.z += __shfl_xor(yv.z, o, LI_WAVE);
+                    yv.w += __shfl_xor(yv.w, o, LI_WAVE);
+                }
+                if (s == 0 && cols)
+                    *reinterpret_cast<float4*>(y + (size_t)(t0 + b0 + tt) * y_stride + (size_t)head * vdim + p) =
+                        float4{fmaf(Dh, xv.x, yv.x), fmaf(Dh, xv.y, yv.y), fmaf(Dh, xv.z, yv.z), fmaf(Dh, xv.w, yv.w)};
+            } else {
+                prod *= a;
+            }
+        }
+    }
+    if (!active) return;
+    float* dst = nullptr;
+    if (MODE == 1) {
+        dst = carry + (size_t)bx * heads * N * vdim + hoff;
+        if (lane == 0 && pbase == 0) decay[(size_t)bx * heads + head] = prod;
+    } else if (last) {
+        dst = state + (size_t)slots[seg] * heads * N * vdim + hoff;
+    }
+    if (dst && cols) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int n = s * NR + r;
+            if (n < N) *reinterpret_cast<float4*>(dst + (size_t)n * vdim + p) = S[r];
+        }
+    }
+}
+
 // Numbers the chunks of a step: request after request, chunk after chunk.  chunk_first[seg] is a request's
 // first chunk; chunk_seg / chunk_idx say whose chunk, and which of its chunks, a number is (-1: none).
 __global__ __launch_bounds__(256) void ssm_chunk_index_kernel(const int* __restrict__ q_len, int segs, int Q, int max_chunks,
@@ -236,17 +375,18 @@ __global__ __launch_bounds__(256) void ssm_carry_kernel(float* __restrict__ carr
     }
 }
 
-template <int NR, int NS>
+template <int NR, int NS, bool QUAD>
 static int ssm_launch(const float* xbc, long xbc_stride, const float* dt_raw, long dt_stride, const float* dt_bias,
                       const float* A_log, const float* Dw, float* state, const int* slots, const int* q_start, const int* q_len,
                       int* chunk_tab, float* carry, float* decay, float* y, long y_stride, int heads, int vdim, int N, int G,
                       int Q, int segs, int max_chunks, bool chunked, hipStream_t stream) {
-    constexpr int NP = NR * NS, PW = 64 / NS;
+    constexpr int NP = NR * NS, PW = (QUAD ? 256 : 64) / NS;
     const size_t lds = (size_t)(2 * SSM_TB * NP + SSM_WAVES * SSM_TB * PW + 2 * SSM_WAVES * SSM_TB) * sizeof(float);
+#define SSM_KERNEL(MODE_) (QUAD ? ssm_scan_quad_kernel<(QUAD ? NR : 4), (QUAD ? NS : 2), MODE_> : ssm_scan_kernel<(QUAD ? 16 : NR), (QUAD ? 1 : NS), MODE_>)
     const int hpg = heads / G, PS = (vdim + PW - 1) / PW, U = hpg * PS, ublocks = (U + SSM_WAVES - 1) / SSM_WAVES;
     if (!chunked) {
         const dim3 grid(segs, G * ublocks);
-        ssm_scan_kernel<NR, NS, 0><<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
+        SSM_KERNEL(0)<<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
             state, slots, q_start, q_len, nullptr, nullptr, nullptr, nullptr, y, y_stride, heads, vdim, N, G, Q);
         return li_launch_status();
     }
@@ -255,15 +395,31 @@ static int ssm_launch(const float* xbc, long xbc_stride, const float* dt_raw, lo
     int* chunk_first = chunk_tab + 2 * max_chunks;
     ssm_chunk_index_kernel<<<1, 256, 0, stream>>>(q_len, segs, Q, max_chunks, chunk_seg, chunk_idx, chunk_first);
     const dim3 grid(max_chunks, G * ublocks);
-    ssm_scan_kernel<NR, NS, 1><<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
+    SSM_KERNEL(1)<<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
         state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q);
     const int NV = N * vdim;
     int zs = (NV + 255) / 256;
     if (zs > 16) zs = 16;
     ssm_carry_kernel<<<dim3(segs, heads, zs), 256, 0, stream>>>(carry, decay, state, slots, q_len, chunk_first, heads, NV, Q);
-    ssm_scan_kernel<NR, NS, 0><<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
+    SSM_KERNEL(0)<<<grid, 64 * SSM_WAVES, lds, stream>>>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw,
         state, slots, q_start, q_len, chunk_seg, chunk_idx, carry, decay, y, y_stride, heads, vdim, N, G, Q);
     return li_launch_status();
+#undef SSM_KERNEL
+}
+
+// The four-columns-a-lane layout for a state of N values a column and heads of vdim columns (a multiple of 4): lanes
+// a quad of columns (2 to 16) and values a lane and column (4 to 32); 0 if it has none.
+static int ssm_quad_layout(int N, int vdim, int* slices, int* per_lane) {
+    if (N <= 0 || N > 256 || vdim <= 0 || vdim % 4) return 0;
+    int ns = 2;
+    while (ns < 16 && 256 / (2 * ns) >= vdim) ns *= 2;      // narrow heads: more lanes a quad, so that a wave is full
+    while (ns < 16 && (N + ns - 1) / ns > 32) ns *= 2;      // at most 32 values a lane and column (128 registers)
+    const int need = (N + ns - 1) / ns;
+    const int nr = need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16 : need <= 32 ? 32 : 0;
+    if (!nr || ns * nr > 256) return 0;
+    *slices = ns;
+    *per_lane = nr;
+    return 1;
 }
 
 // How a state of N values a column is spread: slices (lanes a column) and values a lane; 0 if no kernel has it.
@@ -316,9 +472,22 @@ extern "C" int li_ssm_scan(const float* xbc, long xbc_stride, const float* dt_ra
         carry = (float*)work + ints;
         decay = carry + (size_t)max_chunks * heads * N * vdim;
     }
+    const bool aligned = ((uintptr_t)state | (uintptr_t)y | (uintptr_t)carry) % 16 == 0 && y_stride % 4 == 0;
+    int qs = 0, qr = 0;
+    if (aligned && ssm_quad_layout(N, vdim, &qs, &qr)) {
+#define SSM_QUAD(NR_, NS_)                                                                                                \
+    if (qr == NR_ && qs == NS_)                                                                                           \
+        return ssm_launch<NR_, NS_, true>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw, state, slots, q_start, q_len, \
+                                          chunk_tab, carry, decay, y, y_stride, heads, vdim, N, G, Q, segs, max_chunks, chunked, stream);
+        SSM_QUAD(4, 2) SSM_QUAD(8, 2) SSM_QUAD(16, 2) SSM_QUAD(32, 2)
+        SSM_QUAD(4, 4) SSM_QUAD(8, 4) SSM_QUAD(16, 4) SSM_QUAD(32, 4)
+        SSM_QUAD(4, 8) SSM_QUAD(8, 8) SSM_QUAD(16, 8) SSM_QUAD(32, 8)
+        SSM_QUAD(4, 16) SSM_QUAD(8, 16) SSM_QUAD(16, 16) SSM_QUAD(32, 16)
+#undef SSM_QUAD
+    }
 #define SSM_GO(NR_, NS_)                                                                                                  \
     if (nr == NR_ && ns == NS_)                                                                                           \
-        return ssm_launch<NR_, NS_>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw, state, slots, q_start, q_len,    \
+        return ssm_launch<NR_, NS_, false>(xbc, xbc_stride, dt_raw, dt_stride, dt_bias, A_log, Dw, state, slots, q_start, q_len,    \
                                     chunk_tab, carry, decay, y, y_stride, heads, vdim, N, G, Q, segs, max_chunks, chunked, stream);
     SSM_GO(16, 1) SSM_GO(32, 1) SSM_GO(64, 1) SSM_GO(128, 1)
     SSM_GO(16, 2) SSM_GO(32, 2) SSM_GO(64, 2) SSM_GO(128, 2)
