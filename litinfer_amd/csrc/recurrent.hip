@@ -12,7 +12,7 @@
 __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     const float* __restrict__ u, long u_stride, int C, int taps, const float* __restrict__ w, const float* __restrict__ b,
     const float* __restrict__ tail, const int* __restrict__ seg_of_token, const int* __restrict__ q_start,
-    const int* __restrict__ slots, float* __restrict__ out, long out_stride) {
+    const int* __restrict__ slots, float* __restrict__ out, long out_stride, float* __restrict__ tail_out) {
     const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
     if (c >= C) return;
     const int seg = seg_of_token[t], i = t - q_start[seg], slot = slots[seg];
@@ -22,6 +22,9 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
         const float v = li >= 0 ? u[(size_t)(t - back) * u_stride + c]
                                 : tail[((size_t)slot * (taps - 1) + (taps - 1 + li)) * C + c];
         acc = fmaf(w[(size_t)c * taps + j], v, acc);
+        // every request brings one token (tail_out is given then): the thread owns the request's channel and moves
+        // its tail up by one as it goes (it has read place j, and will read place j + 1 next)
+        if (tail_out && j > 0) tail_out[((size_t)slot * (taps - 1) + (j - 1)) * C + c] = v;
     }
     out[(size_t)t * out_stride + c] = acc / (1.0f + expf(-acc));
 }
@@ -44,11 +47,13 @@ __global__ __launch_bounds__(256) void conv_tail_update_kernel(
 
 extern "C" int li_causal_conv_silu(const float* u, long u_stride, int C, int taps, const float* w, const float* b, float* tail,
                                    const int* seg_of_token, const int* q_start, const int* q_len, const int* slots,
-                                   float* out, long out_stride, int T, int segs, hipStream_t stream) {
-    if (T <= 0 || segs <= 0 || C <= 0 || taps <= 0 || taps > 64 || u_stride < C || out_stride < C) return LI_ERR_SIZE;
+                                   float* out, long out_stride, int T, int segs, int max_q_len, hipStream_t stream) {
+    if (T <= 0 || segs <= 0 || C <= 0 || taps <= 0 || taps > 64 || u_stride < C || out_stride < C || max_q_len <= 0) return LI_ERR_SIZE;
     const dim3 grid(T, (C + 255) / 256);
-    causal_conv_silu_kernel<<<grid, 256, 0, stream>>>(u, u_stride, C, taps, w, b, tail, seg_of_token, q_start, slots, out, out_stride);
-    if (taps > 1) {
+    const bool single = max_q_len == 1 && taps > 1;            // a decoding step: one kernel does both
+    causal_conv_silu_kernel<<<grid, 256, 0, stream>>>(u, u_stride, C, taps, w, b, tail, seg_of_token, q_start, slots, out, out_stride,
+                                                      single ? tail : nullptr);
+    if (taps > 1 && !single) {
         const dim3 g2(segs, (C + 255) / 256);
         conv_tail_update_kernel<<<g2, 256, 0, stream>>>(u, u_stride, C, taps, tail, q_start, q_len, slots);
     }

@@ -50,7 +50,7 @@ _SIGNATURES = {
         "li_diff_combine": [P, P, I, F, F, F, P, I, L, I],
     },
     "recurrent": {
-        "li_causal_conv_silu": [P, L, I, I, P, P, P, P, P, P, P, P, L, I, I],
+        "li_causal_conv_silu": [P, L, I, I, P, P, P, P, P, P, P, P, L, I, I, I],
         "li_ssm_scan": [P, L, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, P, L],
         "li_gated_group_norm": [P, L, P, L, P, F, P, I, L, I, I, I],
     },
@@ -1385,7 +1385,7 @@ def causal_conv_silu(u: torch.Tensor, w: torch.Tensor, b: Optional[torch.Tensor]
     if t:
         _run("recurrent", "li_causal_conv_silu", u.data_ptr(), u.stride(0), c, taps, w.data_ptr(), 0 if b is None else b.data_ptr(),
              tail.data_ptr(), ctx.seg_of_token.data_ptr(), ctx.q_start.data_ptr(), ctx.q_len.data_ptr(), ctx.state_slots.data_ptr(),
-             out.data_ptr(), out.stride(0), t, ctx.num_segments)
+             out.data_ptr(), out.stride(0), t, ctx.num_segments, int(ctx.max_q_len))
 
 
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d: torch.Tensor,
