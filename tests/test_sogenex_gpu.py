@@ -87,6 +87,48 @@ def test_float32_logits_do_not_depend_on_the_schedule(models, name):
             assert schedules.rel_err(outs[kind][r], outs["whole"][r].astype(np.float64)) < 2e-5, (kind, r)
 
 
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", ["recurrent only", "attention only"])
+def test_models_of_one_kind_of_mixer(tmp_path, dt, kind):
+    """No page group at all (every layer keeps state of fixed size only), and no state at all (recorded steps are then
+    filled up with copies of their last entry): the mixed schedule with eight requests on four slots, and decoding."""
+    if kind == "recurrent only":
+        layers = [cases.mamba_layer(2, 20, 12, 2, 3, 1, cases.moe(3, 2, 24, 0)), cases.mamba_layer(4, 8, 40, 1, 1, 2, None),
+                  cases.mamba_layer(2, 20, 12, 2, 3, 1, cases.moe(3, 2, 24, 0), weights_of=0)]
+    else:
+        layers = [cases.attention_layer(2, 1, 8, 24, 9, 0.0, 0.3, cases.moe(2, 1, 16, 8)), cases.attention_layer(3, 3, 10, 6, 1, 0.5, 0.3, None)]
+    cfg = {"architecture": "Sogenex", "vocab": 50, "width": 40, "norm": {"eps": 1e-6}, "logit_softcap": 5.0, "layers": layers}
+    w32 = cases.draw_weights(cfg, 12)
+    d = cases.write_model(tmp_path / "m", cfg, w32, DT[dt])
+    w = cases.stored(w32, DT[dt])
+    reqs = helpers.random_requests(50, [9, 30, 70, 3, 1, 25, 12, 40], 6)
+    ref = {r: plain.forward(cfg, w, t) for r, t in reqs.items()}
+    for name in ("mixed", "tail"):
+        steps = getattr(schedules, name)(reqs)
+        eng = _engine(d, dt, 8, schedules.max_live_tokens(reqs, steps, 8 if name == "mixed" else 64))
+        assert len(eng.cache.groups) == (0 if kind == "recurrent only" else 2) and eng.cache.has_state == (kind == "recurrent only")
+        out = schedules.run(eng, reqs, steps)
+        eng.cache.check_invariants()
+        check_rows(out, ref, dt, f"{kind} {name}")
+    from litinfer_amd.engine import Engine, StepEntry
+    # six requests decoding together: recorded steps of six, filled to eight where no mixer keeps state
+    eng = Engine.from_dir(d, dtype=dt, device=DEV, page_size=8, max_tokens=512, max_seqs=8)
+    rids = list(reqs)[:6]
+    for r in rids:
+        eng.step([StepEntry(r, reqs[r][:1], [])])
+    got = {r: [] for r in rids}
+    for i in range(1, 9):
+        live = [r for r in rids if len(reqs[r]) > i]
+        if not live:
+            break
+        out = eng.step([StepEntry(r, [reqs[r][i]], [0]) for r in live]).float().cpu().numpy()
+        for r, row in zip(live, out):
+            got[r].append(row.copy())
+    for r in rids:
+        if got[r]:
+            check_rows({r: np.stack(got[r])}, {r: ref[r][1:1 + len(got[r])]}, dt, f"{kind} decoding together {r}")
+
+
 def test_layers_that_share_tensors_keep_caches_and_states_of_their_own(models):
     from litinfer_amd.config import load_config
     d, _, _ = models[("A", "float32")]
@@ -319,7 +361,8 @@ def test_causal_convolution_with_its_tail_across_steps(taps, C):
     assert bool((tail[1] == 7.0).all())
 
 
-@pytest.mark.parametrize("heads,vdim,N,G", [(4, 16, 24, 2), (2, 64, 128, 1), (3, 40, 8, 3), (2, 32, 160, 2), (8, 32, 32, 2), (1, 8, 256, 1)])
+@pytest.mark.parametrize("heads,vdim,N,G", [(4, 16, 24, 2), (2, 64, 128, 1), (3, 40, 8, 3), (2, 32, 160, 2), (8, 32, 32, 2), (1, 8, 256, 1),
+                                            (2, 30, 20, 1), (4, 7, 130, 2), (1, 128, 64, 1)])     # (head sizes that are no multiple of 4: one column a lane)
 def test_state_space_recurrence_in_one_pass_in_chunks_and_across_steps(heads, vdim, N, G):
     from litinfer_amd.kernels import ops
     rng = np.random.default_rng(N + vdim)
