@@ -29,6 +29,36 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     out[(size_t)t * out_stride + c] = acc / (1.0f + expf(-acc));
 }
 
+// The same for many tokens with four neighbouring channels a thread (channels, strides and addresses in multiples of
+// four floats): 16-byte loads and stores; the taps' weights of the four channels lie one after the other.
+template <int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_silu_vec_kernel(
+    const float* __restrict__ u, long u_stride, int C, const float* __restrict__ w, const float* __restrict__ b,
+    const float* __restrict__ tail, const int* __restrict__ seg_of_token, const int* __restrict__ q_start,
+    const int* __restrict__ slots, float* __restrict__ out, long out_stride) {
+    const int t = blockIdx.x, c = 4 * (blockIdx.y * 256 + threadIdx.x);
+    if (c >= C) return;
+    const int seg = seg_of_token[t], i = t - q_start[seg], slot = slots[seg];
+    float4 acc = b ? *reinterpret_cast<const float4*>(b + c) : float4{0.f, 0.f, 0.f, 0.f};
+    float wv[4][TAPS];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) wv[k][j] = w[(size_t)(c + k) * TAPS + j];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+        const int back = TAPS - 1 - j, li = i - back;
+        const float4 v = *reinterpret_cast<const float4*>(li >= 0 ? u + (size_t)(t - back) * u_stride + c
+                                                                  : tail + ((size_t)slot * (TAPS - 1) + (TAPS - 1 + li)) * C + c);
+        acc.x = fmaf(wv[0][j], v.x, acc.x);
+        acc.y = fmaf(wv[1][j], v.y, acc.y);
+        acc.z = fmaf(wv[2][j], v.z, acc.z);
+        acc.w = fmaf(wv[3][j], v.w, acc.w);
+    }
+    *reinterpret_cast<float4*>(out + (size_t)t * out_stride + c) =
+        float4{acc.x / (1.0f + expf(-acc.x)), acc.y / (1.0f + expf(-acc.y)), acc.z / (1.0f + expf(-acc.z)), acc.w / (1.0f + expf(-acc.w))};
+}
+
 // The tail after the step: the last taps - 1 inputs of the request, those of this portion and, where it is
 // shorter than that, what is left of the old tail.  A thread owns a (request, channel) and goes upwards, so
 // it never reads what it has written.
@@ -51,8 +81,18 @@ extern "C" int li_causal_conv_silu(const float* u, long u_stride, int C, int tap
     if (T <= 0 || segs <= 0 || C <= 0 || taps <= 0 || taps > 64 || u_stride < C || out_stride < C || max_q_len <= 0) return LI_ERR_SIZE;
     const dim3 grid(T, (C + 255) / 256);
     const bool single = max_q_len == 1 && taps > 1;            // a decoding step: one kernel does both
-    causal_conv_silu_kernel<<<grid, 256, 0, stream>>>(u, u_stride, C, taps, w, b, tail, seg_of_token, q_start, slots, out, out_stride,
-                                                      single ? tail : nullptr);
+    const bool vec = !single && T >= 64 && taps >= 2 && taps <= 4 && C % 4 == 0 && u_stride % 4 == 0 && out_stride % 4 == 0 &&
+                     ((uintptr_t)u | (uintptr_t)out | (uintptr_t)tail | (uintptr_t)b) % 16 == 0;
+    const dim3 grid4(T, (C / 4 + 255) / 256);
+    if (vec && taps == 2)
+        causal_conv_silu_vec_kernel<2><<<grid4, 256, 0, stream>>>(u, u_stride, C, w, b, tail, seg_of_token, q_start, slots, out, out_stride);
+    else if (vec && taps == 3)
+        causal_conv_silu_vec_kernel<3><<<grid4, 256, 0, stream>>>(u, u_stride, C, w, b, tail, seg_of_token, q_start, slots, out, out_stride);
+    else if (vec)
+        causal_conv_silu_vec_kernel<4><<<grid4, 256, 0, stream>>>(u, u_stride, C, w, b, tail, seg_of_token, q_start, slots, out, out_stride);
+    else
+        causal_conv_silu_kernel<<<grid, 256, 0, stream>>>(u, u_stride, C, taps, w, b, tail, seg_of_token, q_start, slots, out, out_stride,
+                                                          single ? tail : nullptr);
     if (taps > 1 && !single) {
         const dim3 g2(segs, (C + 255) / 256);
         conv_tail_update_kernel<<<g2, 256, 0, stream>>>(u, u_stride, C, taps, tail, q_start, q_len, slots);

@@ -336,23 +336,25 @@ def _ctx(q_lens, slots):
                            state_slots=dev(slots), max_q_len=int(q_len.max()))
 
 
-@pytest.mark.parametrize("taps,C", [(4, 37), (2, 300), (7, 64)])
+@pytest.mark.parametrize("taps,C", [(4, 37), (2, 300), (7, 64), (4, 128), (3, 72)])
 def test_causal_convolution_with_its_tail_across_steps(taps, C):
     from litinfer_amd.kernels import ops
     rng = np.random.default_rng(taps)
     w, b = rng.normal(size=(C, taps)), rng.normal(size=C)
-    seqs = {0: rng.normal(size=(40, C)), 2: rng.normal(size=(23, C))}              # by state slot
+    seqs = {0: rng.normal(size=(140, C)), 2: rng.normal(size=(124, C))}            # by state slot
     ref = {s: plain.silu(plain.causal_conv(u, w, b)) for s, u in seqs.items()}
     tail = torch.zeros(3, taps - 1, C, device=DEV)
     tail[1] = 7.0                                                                  # a slot nobody uses stays as it is
     wd, bd = torch.tensor(w, dtype=torch.float32, device=DEV), torch.tensor(b, dtype=torch.float32, device=DEV)
     at = {0: 0, 2: 0}
-    for step in ([(0, 1), (2, 5)], [(2, 1), (0, 2)], [(0, 1)], [(0, 20), (2, 2)], [(2, 15), (0, 16)]):      # (slot, tokens)
+    # (slot, tokens); the last step has rows enough for the form with four channels a thread, where the sizes allow it
+    for k, step in enumerate(([(0, 1), (2, 5)], [(2, 1), (0, 2)], [(0, 1)], [(0, 20), (2, 2)], [(2, 15), (0, 16)], [(2, 100), (0, 1), ], [(0, 99), (2, 1)])):
         u = np.concatenate([seqs[s][at[s]:at[s] + n] for s, n in step])
-        wide = torch.zeros(len(u), C + 5, device=DEV)                               # the rows are a view with a stride
-        wide[:, 3:3 + C] = torch.tensor(u, dtype=torch.float32)
+        lead, extra = (4, 8) if k >= 5 else (3, 5)                                  # the rows are a view with a stride
+        wide = torch.zeros(len(u), C + extra, device=DEV)
+        wide[:, lead:lead + C] = torch.tensor(u, dtype=torch.float32)
         out = torch.empty(len(u), C, device=DEV)
-        ops.causal_conv_silu(wide[:, 3:3 + C], wd, bd, tail, _ctx([n for _, n in step], [s for s, _ in step]), out)
+        ops.causal_conv_silu(wide[:, lead:lead + C], wd, bd, tail, _ctx([n for _, n in step], [s for s, _ in step]), out)
         o = 0
         for s, n in step:
             np.testing.assert_allclose(out[o:o + n].cpu().numpy(), ref[s][at[s]:at[s] + n], rtol=2e-5, atol=2e-5)
