@@ -6,6 +6,7 @@
 #include "common.h"
 
 #define MOE_TILE 32            // rows of one expert that a tile holds
+#define MOE_BIG_TILE 64        // ... where experts get hundreds of rows each (a prompt's portion): the tiles of the LDS kernel
 
 // ------------------------------------------------------------------------------------------------ router
 // One block a token.  logits[e] = b[e] + sum_k W[e, k] x[k] in float32 (a wave an expert, in turns); the `top`
@@ -118,7 +119,8 @@ extern "C" int li_moe_route(const void* x, int x_dtype, long x_stride, const voi
 // together), and the tiles: (expert, first row, rows).  plan = [n_tiles, 0, 0, 0 | tiles x 4 | ...]; row_token[row] is
 // the token of a sorted row, pair_row[pair] the row of pair = token * top + choice.
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ idx, int pairs, int top, int E, int* __restrict__ plan,
-                                                        int max_tiles, int* __restrict__ row_token, int* __restrict__ pair_row) {
+                                                        int max_tiles, int* __restrict__ row_token, int* __restrict__ pair_row,
+                                                        int tile_rows) {
     extern __shared__ int si[];                         // [E] counts, then cursors; [E + 1] starts
     int* cnt = si;
     int* start = si + E;
@@ -133,9 +135,9 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
         int at = 0, nt = 0;
         for (int e = 0; e < E; ++e) {
             start[e] = at;
-            for (int r = 0; r < cnt[e] && nt < max_tiles; r += MOE_TILE, ++nt) {
+            for (int r = 0; r < cnt[e] && nt < max_tiles; r += tile_rows, ++nt) {
                 int* tile = plan + 4 + 4 * nt;
-                tile[0] = e; tile[1] = at + r; tile[2] = (cnt[e] - r < MOE_TILE) ? cnt[e] - r : MOE_TILE; tile[3] = 0;
+                tile[0] = e; tile[1] = at + r; tile[2] = (cnt[e] - r < tile_rows) ? cnt[e] - r : tile_rows; tile[3] = 0;
             }
             at += cnt[e];
         }
@@ -160,9 +162,9 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
 }
 
 extern "C" int li_moe_plan(const int* idx, int T, int top, int E, int* plan, int max_tiles, int* row_token, int* pair_row,
-                           hipStream_t stream) {
-    if (T <= 0 || top <= 0 || E <= 0 || E > 8000 || max_tiles <= 0) return LI_ERR_SIZE;
-    moe_plan_kernel<<<1, 1024, (size_t)(2 * E + 1) * 4, stream>>>(idx, T * top, top, E, plan, max_tiles, row_token, pair_row);
+                           int tile_rows, hipStream_t stream) {
+    if (T <= 0 || top <= 0 || E <= 0 || E > 8000 || max_tiles <= 0 || (tile_rows != MOE_TILE && tile_rows != MOE_BIG_TILE)) return LI_ERR_SIZE;
+    moe_plan_kernel<<<1, 1024, (size_t)(2 * E + 1) * 4, stream>>>(idx, T * top, top, E, plan, max_tiles, row_token, pair_row, tile_rows);
     return li_launch_status();
 }
 
@@ -412,10 +414,144 @@ __global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restri
     }
 }
 
+// Many rows an expert (tiles of up to 64 rows): a block takes a tile and 128 outputs, K in steps of 32 through LDS, so
+// that a matrix row that came from memory serves 64 rows and a token's row 128 outputs; its four waves are two by two,
+// each with 32 rows x 64 outputs (two accumulators).  The block is small on purpose: five or more of them share a compute
+// unit, and while one waits for its next pieces (they wait in registers while this step is multiplied) or at its
+// barriers, the others multiply.  bfloat16 rows and matrices; the same transposed tiles (outputs x rows) as above.
+#define MB_ROWS MOE_BIG_TILE
+#define MB_COLS 128
+#define MB_K 32                // k-values a step (64 bytes of a row: with 128 a block's LDS doubles and half as many blocks share a compute unit: 298 against 210 us)
+#define MB_LD (MB_K + 8)       // elements of an LDS row: 8 of padding (144 bytes: the 16-byte reads of 16 lanes spread over the banks)
+
+template <typename TO>
+__global__ __launch_bounds__(256) void moe_linear_lds_kernel(const bf16_t* __restrict__ a, long a_stride, const int* __restrict__ row_token,
+                                                             const bf16_t* __restrict__ w, const int* __restrict__ plan,
+                                                             TO* __restrict__ out, long out_stride, int n_out, int K, int act,
+                                                             int max_tiles) {
+    __shared__ __align__(16) uint16_t As[MB_ROWS * MB_LD];
+    __shared__ __align__(16) uint16_t Ws[MB_COLS * MB_LD];
+    __shared__ int src[MB_ROWS];
+    // (eight tiles that follow each other against the same columns go to one XCD: see the wide kernel)
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int item = (((idx >> 3) << 3) + xcd) * 8 + (idx & 7);
+    const int cb = item / max_tiles, tile = item % max_tiles;
+    if (tile >= plan[0] || cb * MB_COLS >= n_out) return;
+    const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, ql = lane & 31, h2 = lane >> 5;
+    const int j0 = cb * MB_COLS;
+    if (tid < MB_ROWS) {
+        const int r = r0 + (tid < nr ? tid : nr - 1);
+        src[tid] = row_token ? row_token[r] : r;
+    }
+    __syncthreads();
+    // what a thread brings in a step: 16-byte pieces, MB_K / 8 to a row: NA of token rows, NW of matrix rows
+    constexpr int PP = MB_K / 8, RP = 256 / PP, NA = MB_ROWS / RP, NW = MB_COLS / RP;
+    const int prow = tid / PP, part = tid % PP;
+    const bf16_t* ga[NA];
+    const bf16_t* gw[NW];
+    int la[NA], lw[NW];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        const int row = prow + RP * i;
+        ga[i] = a + (size_t)src[row] * a_stride + 8 * part;
+        la[i] = row * MB_LD + 8 * part;
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+        const int row = prow + RP * i;
+        const int j = j0 + row < n_out ? j0 + row : n_out - 1;
+        gw[i] = w + ((size_t)e * n_out + j) * K + 8 * part;
+        lw[i] = row * MB_LD + 8 * part;
+    }
+    const int wr = wv >> 1, wc = wv & 1;               // the wave's 32 rows and 64 outputs
+    moe_f32x16 acc[2];
+#pragma unroll
+    for (int cf = 0; cf < 2; ++cf)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[cf][i] = 0.f;
+    // the pieces of the next TWO steps wait in registers: a step's pieces are asked for two steps before they go to LDS
+    uint4 ra[2][NA], rw[2][NW];
+    const int last = K - MB_K;
+#pragma unroll
+    for (int d = 0; d < 2; ++d) {
+        const int kd = d * MB_K < last ? d * MB_K : last;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) ra[d][i] = *reinterpret_cast<const uint4*>(ga[i] + kd);
+#pragma unroll
+        for (int i = 0; i < NW; ++i) rw[d][i] = *reinterpret_cast<const uint4*>(gw[i] + kd);
+    }
+    for (int k = 0; k < K; k += MB_K) {
+        __syncthreads();                               // the step before has been read
+#pragma unroll
+        for (int i = 0; i < NA; ++i) *reinterpret_cast<uint4*>(&As[la[i]]) = ra[0][i];
+#pragma unroll
+        for (int i = 0; i < NW; ++i) *reinterpret_cast<uint4*>(&Ws[lw[i]]) = rw[0][i];
+        __syncthreads();
+        const int kn = k + 2 * MB_K < last ? k + 2 * MB_K : last;      // (past the end: the last step again, no branch around the loads)
+#pragma unroll
+        for (int i = 0; i < NA; ++i) { ra[0][i] = ra[1][i]; ra[1][i] = *reinterpret_cast<const uint4*>(ga[i] + kn); }
+#pragma unroll
+        for (int i = 0; i < NW; ++i) { rw[0][i] = rw[1][i]; rw[1][i] = *reinterpret_cast<const uint4*>(gw[i] + kn); }
+#pragma unroll
+        for (int s2 = 0; s2 < MB_K / 16; ++s2) {
+            moe_frag8 fa, fw[2];
+            fa.raw = *reinterpret_cast<const uint4*>(&As[(32 * wr + ql) * MB_LD + 16 * s2 + 8 * h2]);
+#pragma unroll
+            for (int cf = 0; cf < 2; ++cf)
+                fw[cf].raw = *reinterpret_cast<const uint4*>(&Ws[(64 * wc + 32 * cf + ql) * MB_LD + 16 * s2 + 8 * h2]);
+#pragma unroll
+            for (int cf = 0; cf < 2; ++cf) acc[cf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[cf].v, fa.v, acc[cf], 0, 0, 0);
+        }
+    }
+    const int row = 32 * wr + ql;
+    if (row >= nr) return;
+    TO* orow = out + (size_t)(r0 + row) * out_stride + j0 + 64 * wc;
+#pragma unroll
+    for (int cf = 0; cf < 2; ++cf) {
+        if (j0 + 64 * wc + 32 * cf >= n_out) continue;
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {               // registers 4 rg .. 4 rg + 3: outputs 32 cf + 8 rg + 4 h2 ..
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i] = acc[cf][4 * rg + i];
+                if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
+            }
+            TO* dst = orow + 32 * cf + 8 * rg + 4 * h2;
+            if constexpr (sizeof(TO) == 2) {
+                uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
+                d2[0] = pack2_bf16(v[0], v[1]);
+                d2[1] = pack2_bf16(v[2], v[3]);
+            } else {
+                *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+            }
+        }
+    }
+}
+
+// 1 if tiles of MOE_BIG_TILE rows have a kernel for these operands
+extern "C" int li_moe_linear_big_takes(int a_dtype, int w_dtype, int n_out, int K) {
+    return a_dtype == LI_BF16 && w_dtype == LI_BF16 && K % MB_K == 0 && n_out % 32 == 0;
+}
+
 extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const int* row_token, const void* w, int w_dtype,
                              const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act,
-                             hipStream_t stream) {
+                             int tile_rows, hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || out_stride < n_out || act < 0 || act > 1) return LI_ERR_SIZE;
+    if (tile_rows == MOE_BIG_TILE) {
+        if (!li_moe_linear_big_takes(a_dtype, w_dtype, n_out, K) || a_stride % 8 || out_stride % 4 ||
+            ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16)
+            return LI_ERR_SIZE;
+        const dim3 line((unsigned)((((long)max_tiles * ((n_out + MB_COLS - 1) / MB_COLS) + 63) / 64) * 64));
+        if (out_dtype == LI_BF16)
+            moe_linear_lds_kernel<bf16_t><<<line, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (bf16_t*)out, out_stride, n_out, K, act, max_tiles);
+        else if (out_dtype == LI_F32)
+            moe_linear_lds_kernel<float><<<line, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (float*)out, out_stride, n_out, K, act, max_tiles);
+        else return LI_ERR_DTYPE;
+        return li_launch_status();
+    }
+    if (tile_rows != MOE_TILE) return LI_ERR_SIZE;
     if (w_dtype == LI_BF16 && K % 16 == 0 && n_out % 32 == 0 && a_stride % 8 == 0 && out_stride % 4 == 0 &&
         ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0 && (a_dtype == LI_BF16 || a_dtype == LI_F32)) {
         // few tiles (a decoding step: each streams its expert's whole matrix): K in quarters over a block's waves

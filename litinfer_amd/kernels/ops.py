@@ -56,8 +56,8 @@ _SIGNATURES = {
     },
     "moe": {
         "li_moe_route": [P, I, L, P, I, P, P, P, P, P, I, I, I, I],
-        "li_moe_plan": [P, I, I, I, P, I, P, P],
-        "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I],
+        "li_moe_plan": [P, I, I, I, P, I, P, P, I],
+        "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I, I],
         "li_moe_combine": [P, L, P, L, P, P, P, P, L, I, I, I],
     },
     "attention_masked": {
@@ -1434,10 +1434,23 @@ def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps
 MOE_TILE_ROWS = 32       # rows of one expert that a block of the products takes
 
 
-def moe_max_tiles(tokens: int, top: int, experts: int) -> int:
+MOE_BIG_TILE_ROWS = 64   # ... where the experts get hundreds of rows each (a prompt's portion)
+
+
+def moe_tile_rows(tokens: int, top: int, experts: int, a_dtype, w_dtype, sizes) -> int:
+    """Rows a tile for a step of this many tokens: the large tiles where every expert gets twice their rows on average
+    and the kernel that takes them has these operands (`sizes`: (n_out, K) of every product)."""
+    takes = _lib_fn("moe", "li_moe_linear_big_takes", [c_int] * 4, c_int)
+    if tokens * top >= 2 * MOE_BIG_TILE_ROWS * experts and a_dtype in _DT and w_dtype in _DT and all(
+            takes(_DT[a_dtype], _DT[w_dtype], int(n), int(k)) for n, k in sizes):
+        return MOE_BIG_TILE_ROWS
+    return MOE_TILE_ROWS
+
+
+def moe_max_tiles(tokens: int, top: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> int:
     """The most tiles a step can have: every expert's rows end in a tile that may not be full."""
     pairs = tokens * top
-    return min(pairs, pairs // MOE_TILE_ROWS + experts)
+    return min(pairs, pairs // tile_rows + experts)
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], gate_row: Optional[torch.Tensor],
@@ -1460,23 +1473,26 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
              0 if gate is None else gate.data_ptr(), t, k, e, top)
 
 
-def moe_plan(idx: torch.Tensor, experts: int, plan: torch.Tensor, row_token: torch.Tensor, pair_row: torch.Tensor) -> int:
+def moe_plan(idx: torch.Tensor, experts: int, plan: torch.Tensor, row_token: torch.Tensor, pair_row: torch.Tensor,
+             tile_rows: int = MOE_TILE_ROWS) -> int:
     """Sorts the (token, choice) pairs by expert.  plan int32 [4 + 4 * max_tiles]: the number of tiles, then (expert,
     first row, rows, 0) a tile; row_token [pairs]: the token of a sorted row; pair_row [pairs]: the row of a pair.
     Returns max_tiles."""
     _gpu(idx, plan, row_token, pair_row)
     t, top = idx.shape
-    max_tiles = moe_max_tiles(t, top, experts)
+    max_tiles = moe_max_tiles(t, top, experts, tile_rows)
+    _chk(tile_rows in (MOE_TILE_ROWS, MOE_BIG_TILE_ROWS), "moe_plan: tiles of 32 or 64 rows")
     _chk(all(x.dtype is torch.int32 and x.is_contiguous() for x in (idx, plan, row_token, pair_row))
          and plan.numel() >= 4 + 4 * max_tiles and row_token.numel() >= t * top and pair_row.numel() >= t * top and experts <= 8000,
          "moe_plan: int32 arrays of the step's sizes")
     if t:
-        _run("moe", "li_moe_plan", idx.data_ptr(), t, top, experts, plan.data_ptr(), max_tiles, row_token.data_ptr(), pair_row.data_ptr())
+        _run("moe", "li_moe_plan", idx.data_ptr(), t, top, experts, plan.data_ptr(), max_tiles, row_token.data_ptr(), pair_row.data_ptr(),
+             int(tile_rows))
     return max_tiles
 
 
 def moe_linear(a: torch.Tensor, row_token: Optional[torch.Tensor], w: torch.Tensor, plan: torch.Tensor, max_tiles: int,
-               out: torch.Tensor, rows: int, act: int = 0) -> None:
+               out: torch.Tensor, rows: int, act: int = 0, tile_rows: int = MOE_TILE_ROWS) -> None:
     """out[row] = act(W[expert of the row's tile] a[src(row)]) for the sorted rows of the plan; src(row) = row_token[row]
     where given (rows gathered from tokens), else the row.  w [experts, n_out, K]; act 1: max(., 0)^2."""
     _gpu(a, row_token, w, plan, out)
@@ -1488,7 +1504,8 @@ def moe_linear(a: torch.Tensor, row_token: Optional[torch.Tensor], w: torch.Tens
          and (row_token is None or (row_token.dtype is torch.int32 and row_token.numel() >= rows)), "moe_linear: plan, rows")
     if rows:
         _run("moe", "li_moe_linear", a.data_ptr(), _DT[a.dtype], a.stride(0), 0 if row_token is None else row_token.data_ptr(),
-             w.data_ptr(), _DT[w.dtype], plan.data_ptr(), int(max_tiles), out.data_ptr(), _DT[out.dtype], out.stride(0), n_out, k, int(act))
+             w.data_ptr(), _DT[w.dtype], plan.data_ptr(), int(max_tiles), out.data_ptr(), _DT[out.dtype], out.stride(0), n_out, k, int(act),
+             int(tile_rows))
 
 
 def moe_combine(x: torch.Tensor, yrows: torch.Tensor, pair_row: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor],

@@ -83,15 +83,18 @@ class RoutedReluSquaredMLP(FeedForward):
         wt = ws.buffer("moe.wt", (t, top), torch.float32)
         gate = ws.buffer("moe.gate", (t,), torch.float32) if self.gate_row is not None else None
         ops.moe_route(xn, self.router, self.router_b, self.gate_row, idx, wt, gate)
-        max_tiles = ops.moe_max_tiles(t, top, self.experts)
+        # (a prompt's portion gives every expert hundreds of rows: larger tiles then, for the kernel that stages them in LDS)
+        rows_a_tile = ops.moe_tile_rows(t, top, self.experts, xn.dtype, self.w_up.dtype,
+                                        ((self.inter, self.hidden), (self.hidden, self.inter)))
+        max_tiles = ops.moe_max_tiles(t, top, self.experts, rows_a_tile)
         plan = ws.buffer("moe.plan", (4 + 4 * max_tiles,), torch.int32)
         row_token = ws.buffer("moe.row_token", (pairs,), torch.int32)
         pair_row = ws.buffer("moe.pair_row", (pairs,), torch.int32)
-        ops.moe_plan(idx, self.experts, plan, row_token, pair_row)
+        ops.moe_plan(idx, self.experts, plan, row_token, pair_row, rows_a_tile)
         h = ws.buffer("moe.h", (pairs, self.inter), self.rt.dtype)
-        ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=1)
+        ops.moe_linear(xn, row_token, self.w_up, plan, max_tiles, h, pairs, act=1, tile_rows=rows_a_tile)
         yrows = ws.buffer("moe.y", (pairs, self.hidden), torch.float32)
-        ops.moe_linear(h, None, self.w_down, plan, max_tiles, yrows, pairs)
+        ops.moe_linear(h, None, self.w_down, plan, max_tiles, yrows, pairs, tile_rows=rows_a_tile)
         shared = None
         if self.shared_inter:
             u = ws.buffer("mlp.up32", (t, self.shared_inter), torch.float32)
