@@ -6,7 +6,8 @@
 #include "common.h"
 
 #define MOE_TILE 32            // rows of one expert that a tile holds
-#define MOE_BIG_TILE 64        // ... where experts get hundreds of rows each (a prompt's portion): the tiles of the LDS kernel
+#define MOE_BIG_TILE 64        // ... where experts get hundreds of rows each (a prompt's portion): the tiles of the LDS kernel,
+#define MOE_HUGE_TILE 128      // and twice that where they get still more
 
 // ------------------------------------------------------------------------------------------------ router
 // One block a token.  logits[e] = b[e] + sum_k W[e, k] x[k] in float32 (a wave an expert, in turns); the `top`
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
 
 extern "C" int li_moe_plan(const int* idx, int T, int top, int E, int* plan, int max_tiles, int* row_token, int* pair_row,
                            int tile_rows, hipStream_t stream) {
-    if (T <= 0 || top <= 0 || E <= 0 || E > 8000 || max_tiles <= 0 || (tile_rows != MOE_TILE && tile_rows != MOE_BIG_TILE)) return LI_ERR_SIZE;
+    if (T <= 0 || top <= 0 || E <= 0 || E > 8000 || max_tiles <= 0 || (tile_rows != MOE_TILE && tile_rows != MOE_BIG_TILE && tile_rows != MOE_HUGE_TILE)) return LI_ERR_SIZE;
     moe_plan_kernel<<<1, 1024, (size_t)(2 * E + 1) * 4, stream>>>(idx, T * top, top, E, plan, max_tiles, row_token, pair_row, tile_rows);
     return li_launch_status();
 }
@@ -419,16 +420,17 @@ __global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restri
 // each with 32 rows x 64 outputs (two accumulators).  The block is small on purpose: five or more of them share a compute
 // unit, and while one waits for its next pieces (they wait in registers while this step is multiplied) or at its
 // barriers, the others multiply.  bfloat16 rows and matrices; the same transposed tiles (outputs x rows) as above.
-#define MB_ROWS MOE_BIG_TILE
 #define MB_COLS 128
 #define MB_K 32                // k-values a step (64 bytes of a row: with 128 a block's LDS doubles and half as many blocks share a compute unit: 298 against 210 us)
+#define MB_DEPTH 2             // steps whose pieces wait in registers (four: no faster)
 #define MB_LD (MB_K + 8)       // elements of an LDS row: 8 of padding (144 bytes: the 16-byte reads of 16 lanes spread over the banks)
 
-template <typename TO>
+template <typename TO, int RF>      // RF: row fragments of 32 a wave (1: tiles of 64 rows, 2: of 128)
 __global__ __launch_bounds__(256) void moe_linear_lds_kernel(const bf16_t* __restrict__ a, long a_stride, const int* __restrict__ row_token,
                                                              const bf16_t* __restrict__ w, const int* __restrict__ plan,
                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act,
                                                              int max_tiles) {
+    constexpr int MB_ROWS = 64 * RF;
     __shared__ __align__(16) uint16_t As[MB_ROWS * MB_LD];
     __shared__ __align__(16) uint16_t Ws[MB_COLS * MB_LD];
     __shared__ int src[MB_ROWS];
@@ -464,17 +466,19 @@ __global__ __launch_bounds__(256) void moe_linear_lds_kernel(const bf16_t* __res
         gw[i] = w + ((size_t)e * n_out + j) * K + 8 * part;
         lw[i] = row * MB_LD + 8 * part;
     }
-    const int wr = wv >> 1, wc = wv & 1;               // the wave's 32 rows and 64 outputs
-    moe_f32x16 acc[2];
+    const int wr = wv >> 1, wc = wv & 1;               // the wave's 32 * RF rows and 64 outputs
+    moe_f32x16 acc[RF][2];
 #pragma unroll
-    for (int cf = 0; cf < 2; ++cf)
+    for (int rf = 0; rf < RF; ++rf)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[cf][i] = 0.f;
-    // the pieces of the next TWO steps wait in registers: a step's pieces are asked for two steps before they go to LDS
-    uint4 ra[2][NA], rw[2][NW];
+        for (int cf = 0; cf < 2; ++cf)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[rf][cf][i] = 0.f;
+    // the pieces of the next MB_DEPTH steps wait in registers: a step's pieces are asked for that many steps before they go to LDS
+    uint4 ra[MB_DEPTH][NA], rw[MB_DEPTH][NW];
     const int last = K - MB_K;
 #pragma unroll
-    for (int d = 0; d < 2; ++d) {
+    for (int d = 0; d < MB_DEPTH; ++d) {
         const int kd = d * MB_K < last ? d * MB_K : last;
 #pragma unroll
         for (int i = 0; i < NA; ++i) ra[d][i] = *reinterpret_cast<const uint4*>(ga[i] + kd);
@@ -488,43 +492,59 @@ __global__ __launch_bounds__(256) void moe_linear_lds_kernel(const bf16_t* __res
 #pragma unroll
         for (int i = 0; i < NW; ++i) *reinterpret_cast<uint4*>(&Ws[lw[i]]) = rw[0][i];
         __syncthreads();
-        const int kn = k + 2 * MB_K < last ? k + 2 * MB_K : last;      // (past the end: the last step again, no branch around the loads)
+        const int kn = k + MB_DEPTH * MB_K < last ? k + MB_DEPTH * MB_K : last;      // (past the end: the last step again, no branch around the loads)
 #pragma unroll
-        for (int i = 0; i < NA; ++i) { ra[0][i] = ra[1][i]; ra[1][i] = *reinterpret_cast<const uint4*>(ga[i] + kn); }
+        for (int i = 0; i < NA; ++i) {
 #pragma unroll
-        for (int i = 0; i < NW; ++i) { rw[0][i] = rw[1][i]; rw[1][i] = *reinterpret_cast<const uint4*>(gw[i] + kn); }
+            for (int d = 0; d + 1 < MB_DEPTH; ++d) ra[d][i] = ra[d + 1][i];
+            ra[MB_DEPTH - 1][i] = *reinterpret_cast<const uint4*>(ga[i] + kn);
+        }
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+#pragma unroll
+            for (int d = 0; d + 1 < MB_DEPTH; ++d) rw[d][i] = rw[d + 1][i];
+            rw[MB_DEPTH - 1][i] = *reinterpret_cast<const uint4*>(gw[i] + kn);
+        }
 #pragma unroll
         for (int s2 = 0; s2 < MB_K / 16; ++s2) {
-            moe_frag8 fa, fw[2];
-            fa.raw = *reinterpret_cast<const uint4*>(&As[(32 * wr + ql) * MB_LD + 16 * s2 + 8 * h2]);
+            moe_frag8 fa[RF], fw[2];
+#pragma unroll
+            for (int rf = 0; rf < RF; ++rf)
+                fa[rf].raw = *reinterpret_cast<const uint4*>(&As[(32 * RF * wr + 32 * rf + ql) * MB_LD + 16 * s2 + 8 * h2]);
 #pragma unroll
             for (int cf = 0; cf < 2; ++cf)
                 fw[cf].raw = *reinterpret_cast<const uint4*>(&Ws[(64 * wc + 32 * cf + ql) * MB_LD + 16 * s2 + 8 * h2]);
 #pragma unroll
-            for (int cf = 0; cf < 2; ++cf) acc[cf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[cf].v, fa.v, acc[cf], 0, 0, 0);
+            for (int rf = 0; rf < RF; ++rf)
+#pragma unroll
+                for (int cf = 0; cf < 2; ++cf)
+                    acc[rf][cf] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[cf].v, fa[rf].v, acc[rf][cf], 0, 0, 0);
         }
     }
-    const int row = 32 * wr + ql;
-    if (row >= nr) return;
-    TO* orow = out + (size_t)(r0 + row) * out_stride + j0 + 64 * wc;
 #pragma unroll
-    for (int cf = 0; cf < 2; ++cf) {
-        if (j0 + 64 * wc + 32 * cf >= n_out) continue;
+    for (int rf = 0; rf < RF; ++rf) {
+        const int row = 32 * RF * wr + 32 * rf + ql;
+        if (row >= nr) continue;
+        TO* orow = out + (size_t)(r0 + row) * out_stride + j0 + 64 * wc;
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {               // registers 4 rg .. 4 rg + 3: outputs 32 cf + 8 rg + 4 h2 ..
-            float v[4];
+        for (int cf = 0; cf < 2; ++cf) {
+            if (j0 + 64 * wc + 32 * cf >= n_out) continue;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                v[i] = acc[cf][4 * rg + i];
-                if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
-            }
-            TO* dst = orow + 32 * cf + 8 * rg + 4 * h2;
-            if constexpr (sizeof(TO) == 2) {
-                uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
-                d2[0] = pack2_bf16(v[0], v[1]);
-                d2[1] = pack2_bf16(v[2], v[3]);
-            } else {
-                *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+            for (int rg = 0; rg < 4; ++rg) {           // registers 4 rg .. 4 rg + 3: outputs 32 cf + 8 rg + 4 h2 ..
+                float v[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    v[i] = acc[rf][cf][4 * rg + i];
+                    if (act == 1) { v[i] = fmaxf(v[i], 0.f); v[i] *= v[i]; }
+                }
+                TO* dst = orow + 32 * cf + 8 * rg + 4 * h2;
+                if constexpr (sizeof(TO) == 2) {
+                    uint32_t* d2 = reinterpret_cast<uint32_t*>(dst);
+                    d2[0] = pack2_bf16(v[0], v[1]);
+                    d2[1] = pack2_bf16(v[2], v[3]);
+                } else {
+                    *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+                }
             }
         }
     }
@@ -539,16 +559,17 @@ extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const in
                              const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act,
                              int tile_rows, hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || out_stride < n_out || act < 0 || act > 1) return LI_ERR_SIZE;
-    if (tile_rows == MOE_BIG_TILE) {
+    if (tile_rows == MOE_BIG_TILE || tile_rows == MOE_HUGE_TILE) {
         if (!li_moe_linear_big_takes(a_dtype, w_dtype, n_out, K) || a_stride % 8 || out_stride % 4 ||
             ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16)
             return LI_ERR_SIZE;
         const dim3 line((unsigned)((((long)max_tiles * ((n_out + MB_COLS - 1) / MB_COLS) + 63) / 64) * 64));
-        if (out_dtype == LI_BF16)
-            moe_linear_lds_kernel<bf16_t><<<line, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (bf16_t*)out, out_stride, n_out, K, act, max_tiles);
-        else if (out_dtype == LI_F32)
-            moe_linear_lds_kernel<float><<<line, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (float*)out, out_stride, n_out, K, act, max_tiles);
+#define ML(TO, RF) moe_linear_lds_kernel<TO, RF><<<line, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (TO*)out, out_stride, n_out, K, act, max_tiles)
+        const bool huge = tile_rows == MOE_HUGE_TILE;
+        if (out_dtype == LI_BF16) { if (huge) ML(bf16_t, 2); else ML(bf16_t, 1); }
+        else if (out_dtype == LI_F32) { if (huge) ML(float, 2); else ML(float, 1); }
         else return LI_ERR_DTYPE;
+#undef ML
         return li_launch_status();
     }
     if (tile_rows != MOE_TILE) return LI_ERR_SIZE;

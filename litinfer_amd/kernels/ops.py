@@ -1434,7 +1434,8 @@ def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps
 MOE_TILE_ROWS = 32       # rows of one expert that a block of the products takes
 
 
-MOE_BIG_TILE_ROWS = 64   # ... where the experts get hundreds of rows each (a prompt's portion)
+MOE_BIG_TILE_ROWS = 64   # ... where the experts get hundreds of rows each (a prompt's portion),
+MOE_HUGE_TILE_ROWS = 128  # and where they get still more
 
 
 def moe_tile_rows(tokens: int, top: int, experts: int, a_dtype, w_dtype, sizes) -> int:
@@ -1443,7 +1444,7 @@ def moe_tile_rows(tokens: int, top: int, experts: int, a_dtype, w_dtype, sizes) 
     takes = _lib_fn("moe", "li_moe_linear_big_takes", [c_int] * 4, c_int)
     if tokens * top >= 2 * MOE_BIG_TILE_ROWS * experts and a_dtype in _DT and w_dtype in _DT and all(
             takes(_DT[a_dtype], _DT[w_dtype], int(n), int(k)) for n, k in sizes):
-        return MOE_BIG_TILE_ROWS
+        return MOE_HUGE_TILE_ROWS if tokens * top >= 2 * MOE_HUGE_TILE_ROWS * experts else MOE_BIG_TILE_ROWS
     return MOE_TILE_ROWS
 
 
@@ -1481,7 +1482,7 @@ def moe_plan(idx: torch.Tensor, experts: int, plan: torch.Tensor, row_token: tor
     _gpu(idx, plan, row_token, pair_row)
     t, top = idx.shape
     max_tiles = moe_max_tiles(t, top, experts, tile_rows)
-    _chk(tile_rows in (MOE_TILE_ROWS, MOE_BIG_TILE_ROWS), "moe_plan: tiles of 32 or 64 rows")
+    _chk(tile_rows in (MOE_TILE_ROWS, MOE_BIG_TILE_ROWS, MOE_HUGE_TILE_ROWS), "moe_plan: tiles of 32, 64 or 128 rows")
     _chk(all(x.dtype is torch.int32 and x.is_contiguous() for x in (idx, plan, row_token, pair_row))
          and plan.numel() >= 4 + 4 * max_tiles and row_token.numel() >= t * top and pair_row.numel() >= t * top and experts <= 8000,
          "moe_plan: int32 arrays of the step's sizes")

@@ -410,7 +410,7 @@ def test_gated_norm_in_groups():
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 @pytest.mark.parametrize("T,K,E,top,ff,shared", [(1, 96, 5, 2, 40, 56), (70, 128, 8, 2, 64, 128), (300, 64, 3, 3, 48, 0),
                                                  (33, 256, 64, 6, 96, 0), (9, 128, 4, 1, 72, 24), (2200, 256, 4, 2, 160, 0),
-                                                 (40, 512, 6, 2, 48, 0), (1500, 128, 4, 2, 192, 64)])
+                                                 (40, 512, 6, 2, 48, 0), (1500, 128, 4, 2, 192, 64), (600, 128, 8, 2, 96, 0)])
 def test_routed_feed_forward(dt, T, K, E, top, ff, shared):
     """The part itself (router, plan, products by tile, weighted sum, gated shared expert) against the plain one, on
     tokens whose choice of experts is not a close call for the rounding of the engine's dtype."""
