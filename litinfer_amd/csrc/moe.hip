@@ -8,6 +8,7 @@
 #define MOE_TILE 32            // rows of one expert that a tile holds
 #define MOE_BIG_TILE 64        // ... where experts get hundreds of rows each (a prompt's portion): the tiles of the LDS kernel,
 #define MOE_HUGE_TILE 128      // and twice that where they get still more
+#define MOE_FEW_ROWS 32        // rows of a step up to which every row is a matrix-vector product of its own
 
 // ------------------------------------------------------------------------------------------------ router
 // One block a token.  logits[e] = b[e] + sum_k W[e, k] x[k] in float32 (a wave an expert, in turns); the `top`
@@ -415,6 +416,82 @@ __global__ __launch_bounds__(256) void moe_linear_wide_kernel(const TA* __restri
     }
 }
 
+// A handful of rows in all (a decoding step of few requests): every tile streams its expert's matrix for one or two
+// rows, so the product is a matrix-vector product a row.  A wave owns four outputs and walks their matrix rows in
+// 16-byte pieces, 64 lanes side by side along K (a kilobyte of a row at a time, all four rows' pieces asked for
+// together), against up to four of the tile's rows at a time; sums in float32, lanes added up at the end.
+#define MR_OUT 4
+#define MR_ROWS 4
+
+template <typename TO>
+__global__ __launch_bounds__(256) void moe_linear_rows_kernel(const bf16_t* __restrict__ a, long a_stride, const int* __restrict__ row_token,
+                                                              const bf16_t* __restrict__ w, const int* __restrict__ plan,
+                                                              TO* __restrict__ out, long out_stride, int n_out, int K, int act) {
+    const int tile = blockIdx.x;
+    if (tile >= plan[0]) return;
+    const int e = plan[4 + 4 * tile], r0 = plan[5 + 4 * tile], nr = plan[6 + 4 * tile];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int j0 = (blockIdx.y * 4 + wv) * MR_OUT;
+    if (j0 >= n_out) return;
+    const bf16_t* wrow[MR_OUT];
+#pragma unroll
+    for (int j = 0; j < MR_OUT; ++j) wrow[j] = w + ((size_t)e * n_out + (j0 + j < n_out ? j0 + j : n_out - 1)) * K;
+    for (int rc = 0; rc < nr; rc += MR_ROWS) {
+        const bf16_t* xrow[MR_ROWS];
+#pragma unroll
+        for (int r = 0; r < MR_ROWS; ++r) {
+            const int row = r0 + (rc + r < nr ? rc + r : nr - 1);
+            xrow[r] = a + (size_t)(row_token ? row_token[row] : row) * a_stride;
+        }
+        float acc[MR_OUT][MR_ROWS];
+#pragma unroll
+        for (int j = 0; j < MR_OUT; ++j)
+#pragma unroll
+            for (int r = 0; r < MR_ROWS; ++r) acc[j][r] = 0.f;
+        for (int i = lane; i < K / 8; i += 64) {
+            uint4 wp[MR_OUT], xp[MR_ROWS];
+#pragma unroll
+            for (int j = 0; j < MR_OUT; ++j) wp[j] = *reinterpret_cast<const uint4*>(wrow[j] + 8 * i);
+#pragma unroll
+            for (int r = 0; r < MR_ROWS; ++r) xp[r] = *reinterpret_cast<const uint4*>(xrow[r] + 8 * i);
+            float xf[MR_ROWS][8];
+#pragma unroll
+            for (int r = 0; r < MR_ROWS; ++r) {
+                const uint32_t u[4] = {xp[r].x, xp[r].y, xp[r].z, xp[r].w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) { xf[r][2 * q] = __uint_as_float(u[q] << 16); xf[r][2 * q + 1] = __uint_as_float(u[q] & 0xffff0000u); }
+            }
+#pragma unroll
+            for (int j = 0; j < MR_OUT; ++j) {
+                const uint32_t u[4] = {wp[j].x, wp[j].y, wp[j].z, wp[j].w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float lo = __uint_as_float(u[q] << 16), hi = __uint_as_float(u[q] & 0xffff0000u);
+#pragma unroll
+                    for (int r = 0; r < MR_ROWS; ++r) acc[j][r] = fmaf(hi, xf[r][2 * q + 1], fmaf(lo, xf[r][2 * q], acc[j][r]));
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < MR_OUT; ++j)
+#pragma unroll
+            for (int r = 0; r < MR_ROWS; ++r) acc[j][r] = wave_sum(acc[j][r]);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < MR_ROWS; ++r) {
+                if (rc + r >= nr) continue;
+#pragma unroll
+                for (int j = 0; j < MR_OUT; ++j) {
+                    if (j0 + j >= n_out) continue;
+                    float v = acc[j][r];
+                    if (act == 1) { v = fmaxf(v, 0.f); v = v * v; }
+                    store_from_float(out + (size_t)(r0 + rc + r) * out_stride + j0 + j, v);
+                }
+            }
+        }
+    }
+}
+
 // Many rows an expert (tiles of up to 64 rows): a block takes a tile and 128 outputs, K in steps of 32 through LDS, so
 // that a matrix row that came from memory serves 64 rows and a token's row 128 outputs; its four waves are two by two,
 // each with 32 rows x 64 outputs (two accumulators).  The block is small on purpose: five or more of them share a compute
@@ -557,7 +634,7 @@ extern "C" int li_moe_linear_big_takes(int a_dtype, int w_dtype, int n_out, int 
 
 extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const int* row_token, const void* w, int w_dtype,
                              const int* plan, int max_tiles, void* out, int out_dtype, long out_stride, int n_out, int K, int act,
-                             int tile_rows, hipStream_t stream) {
+                             int tile_rows, int rows, hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0 || K <= 0 || a_stride < K || out_stride < n_out || act < 0 || act > 1) return LI_ERR_SIZE;
     if (tile_rows == MOE_BIG_TILE || tile_rows == MOE_HUGE_TILE) {
         if (!li_moe_linear_big_takes(a_dtype, w_dtype, n_out, K) || a_stride % 8 || out_stride % 4 ||
@@ -573,6 +650,16 @@ extern "C" int li_moe_linear(const void* a, int a_dtype, long a_stride, const in
         return li_launch_status();
     }
     if (tile_rows != MOE_TILE) return LI_ERR_SIZE;
+    // a handful of rows in all: a matrix-vector product a row (each tile streams its expert's matrix anyway)
+    if (rows <= MOE_FEW_ROWS && a_dtype == LI_BF16 && w_dtype == LI_BF16 && K % 8 == 0 && a_stride % 8 == 0 &&
+        ((uintptr_t)a | (uintptr_t)w) % 16 == 0 && (out_dtype == LI_BF16 || out_dtype == LI_F32)) {
+        const dim3 grid(max_tiles, (n_out + 4 * MR_OUT - 1) / (4 * MR_OUT));
+        if (out_dtype == LI_BF16)
+            moe_linear_rows_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (bf16_t*)out, out_stride, n_out, K, act);
+        else
+            moe_linear_rows_kernel<float><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, row_token, (const bf16_t*)w, plan, (float*)out, out_stride, n_out, K, act);
+        return li_launch_status();
+    }
     if (w_dtype == LI_BF16 && K % 16 == 0 && n_out % 32 == 0 && a_stride % 8 == 0 && out_stride % 4 == 0 &&
         ((uintptr_t)a | (uintptr_t)w | (uintptr_t)out) % 16 == 0 && (a_dtype == LI_BF16 || a_dtype == LI_F32)) {
         // few tiles (a decoding step: each streams its expert's whole matrix): K in quarters over a block's waves

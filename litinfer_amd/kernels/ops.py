@@ -57,7 +57,7 @@ _SIGNATURES = {
     "moe": {
         "li_moe_route": [P, I, L, P, I, P, P, P, P, P, I, I, I, I],
         "li_moe_plan": [P, I, I, I, P, I, P, P, I],
-        "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I, I],
+        "li_moe_linear": [P, I, L, P, P, I, P, I, P, I, L, I, I, I, I, I],
         "li_moe_combine": [P, L, P, L, P, P, P, P, L, I, I, I],
     },
     "attention_masked": {
@@ -1506,7 +1506,7 @@ def moe_linear(a: torch.Tensor, row_token: Optional[torch.Tensor], w: torch.Tens
     if rows:
         _run("moe", "li_moe_linear", a.data_ptr(), _DT[a.dtype], a.stride(0), 0 if row_token is None else row_token.data_ptr(),
              w.data_ptr(), _DT[w.dtype], plan.data_ptr(), int(max_tiles), out.data_ptr(), _DT[out.dtype], out.stride(0), n_out, k, int(act),
-             int(tile_rows))
+             int(tile_rows), int(rows))
 
 
 def moe_combine(x: torch.Tensor, yrows: torch.Tensor, pair_row: torch.Tensor, wt: torch.Tensor, gate: Optional[torch.Tensor],
